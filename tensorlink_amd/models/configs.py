@@ -116,6 +116,9 @@ class ModelConfig:
         if cfg.get("architecture") in ("Senulix", "senulix"):
             from tensorlink_amd.models.senulix import SenulixConfig
             return SenulixConfig.from_dict(cfg, name=name)
+        if cfg.get("architecture") in ("Dizepel", "dizepel"):
+            from tensorlink_amd.models.dizepel import DizepelConfig
+            return DizepelConfig.from_dict(cfg, name=name)
         if "architecture" in cfg and "architectures" not in cfg:
             # our own to_json round-trip (save_hf_checkpoint writes it)
             known = {f.name for f in dataclasses.fields(cls)}

@@ -457,4 +457,7 @@ def _stage_class(config: ModelConfig):
     if config.architecture == "senulix":
         from tensorlink_amd.models.senulix import SenulixStageModel
         return SenulixStageModel
+    if config.architecture == "dizepel":
+        from tensorlink_amd.models.dizepel import DizepelStageModel
+        return DizepelStageModel
     return StageModel

@@ -73,12 +73,15 @@ class LayeredStage(nn.Module):
 @torch.no_grad()
 def load_named_tensors(params: Dict[str, torch.Tensor],
                        names: Dict[str, Tuple[str, int]], ckpt_dir: str,
-                       optional: Iterable[str] = ()) -> int:
+                       optional: Iterable[str] = (),
+                       partial: Dict[str, int] = None) -> int:
     """Fill ``params`` from ``model.safetensors``. ``names`` maps a
     checkpoint tensor to (parameter, row offset — or expert index for a
     stacked 3-d parameter). Strict both ways: an unknown tensor raises and
     so does a parameter left (partly) unfilled, unless listed in
-    ``optional`` and untouched."""
+    ``optional`` and untouched; ``partial`` names parameters that the
+    checkpoint fills only up to the given number of elements (the rest
+    keeps the caller's values)."""
     from safetensors import safe_open
     filled = {k: 0 for k in params}
     loaded = 0
@@ -103,7 +106,9 @@ def load_named_tensors(params: Dict[str, torch.Tensor],
             filled[pname] += t.numel()
             loaded += 1
     optional = set(optional)
-    short = [k for k, n in filled.items() if n != params[k].numel()
+    partial = partial or {}
+    short = [k for k, n in filled.items()
+             if n != partial.get(k, params[k].numel())
              and not (n == 0 and k in optional)]
     if short:
         raise KeyError(f"checkpoint leaves parameters unfilled: {short[:5]}")

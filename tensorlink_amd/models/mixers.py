@@ -464,3 +464,186 @@ class TokenSide(nn.Module):
         g = mx.gelu(self.gate(h), True, table=table, tokens=tokens,
                     table_col=self.col)
         return self.proj(g)
+
+
+# ---------------------------------------------------------------------------
+# blocks of the parallel-mixer family: layer norm without bias, causal
+# input convolution, softmax attention with short convolutions / a learned
+# sink / capped scores whose values are its unrotated keys, a selective
+# state-space (SSD) mixer, the two side by side, and a PolyNorm feed-forward
+# ---------------------------------------------------------------------------
+class LayerNormWeight(nn.Module, _F32Cache):
+    """Weight of a layer norm without bias."""
+
+    def __init__(self, width: int):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(width))
+
+    def w32(self):
+        return self._f32("weight")
+
+
+class CanonConv(nn.Module, _F32Cache):
+    """Causal per-channel convolution over time added to a sublayer's
+    input: h <- h + conv(h), taps [width, K], no bias. Its last K-1 inputs
+    are per-sequence state (``state_shape``)."""
+
+    def __init__(self, width: int, taps: int):
+        super().__init__()
+        self.taps = int(taps)
+        self.weight = nn.Parameter(torch.zeros(width, taps))
+        self.state_shape = (taps - 1, width)
+
+    def w32(self):
+        return self._f32("weight")
+
+
+class ConvSinkAttention(nn.Module, _F32Cache):
+    """Grouped-query softmax attention over the paged pool whose VALUES are
+    its keys before rotation (no value projection). q and k (with biases,
+    added by the caller's fused projection) pass a short causal
+    convolution over time, then rotate-half positions on the first
+    ``rot_dims`` dimensions of every head (optionally with a two-regime
+    frequency scaling, see ``ops.mixers.yarn_freqs``); scores are scaled,
+    optionally capped through tanh, and the softmax denominator holds one
+    learned logit per head (``sink``) that has no key and no value.
+
+    The module owns everything after the input projection; ``in_cols``
+    columns [q | k] of the caller's projection feed it. Per-sequence
+    memory: key pool (rotated), value pool (unrotated) and the last
+    ``conv - 1`` projected rows (``state_shapes``)."""
+
+    kind = "conv_sink_attention"
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 conv: int, scale: float, softcap: float, rot_dims: int,
+                 rot_base: float, rot_scaling: Optional[dict]):
+        super().__init__()
+        assert heads % kv_heads == 0 and rot_dims % 2 == 0 \
+            and rot_dims <= dim
+        self.H, self.G, self.D, self.K = heads, kv_heads, dim, int(conv)
+        self.scale, self.softcap = float(scale), float(softcap or 0.0)
+        self.rot_dims, self.base = int(rot_dims), float(rot_base)
+        self.rot_scaling = dict(rot_scaling) if rot_scaling else None
+        self.q_cols, self.k_cols = heads * dim, kv_heads * dim
+        self.in_cols = self.q_cols + self.k_cols
+        self.bias_cols = self.in_cols
+        self.qk_conv = nn.Parameter(torch.zeros(self.in_cols, self.K))
+        self.sink = nn.Parameter(torch.zeros(heads))
+        self.o_proj = TLLinear(heads * dim, width, bias=False)
+        self.state_shapes = [(self.K - 1, self.in_cols)]
+
+    def cache_spec(self):
+        return {"kind": "kv", "G": self.G, "DK": self.D, "V": self.D}
+
+    def _freqs(self, dev):
+        hit = self.__dict__.get("_fr")
+        if hit is None or hit[0].device != dev:
+            hit = mx.yarn_freqs(self.rot_dims, self.base, self.rot_scaling,
+                                dev)
+            self.__dict__["_fr"] = hit
+        return hit
+
+    def forward(self, proj, col, meta, kpool, vpool, hist):
+        fr, mult = (self._freqs(proj.device) if self.rot_dims
+                    else (None, 1.0))
+        q = mx.conv_rope_rows(proj, col, self.H + self.G, self.D,
+                              self._f32("qk_conv"), hist, meta,
+                              rot_dims=self.rot_dims, freqs=fr, rot_mult=mult,
+                              pool=kpool, raw_pool=vpool, pool_heads=self.G)
+        o = mx.flex_attention(q, kpool, vpool, meta, self.H, self.scale,
+                              softcap=self.softcap,
+                              sink_logits=self._f32("sink"),
+                              out_dtype=proj.dtype)
+        return self.o_proj(o)
+
+
+class SSDMixer(nn.Module, _F32Cache):
+    """Selective state-space mixer with one scalar decay per head
+    (state-space duality form). Columns [z | x | B | C | dt] of the
+    caller's projection feed it (``in_cols``); x, B, C pass a short causal
+    convolution with bias and silu; dt = softplus(dt + dt_bias);
+    S_t = exp(-exp(A_log) dt) S_(t-1) + dt B_t x_t^T, y_t = S_t^T C_t +
+    D x_t; y * silu(z) is RMS-normed in ``norm_groups`` equal parts, times
+    ``norm``, then the output projection. Per-sequence memory: the state
+    [heads, state, vdim] (fp32) and the convolution's last inputs."""
+
+    kind = "ssd"
+
+    def __init__(self, width: int, heads: int, vdim: int, state: int,
+                 groups: int, conv: int, norm_groups: int, eps: float):
+        super().__init__()
+        assert heads % groups == 0 and (heads * vdim) % norm_groups == 0
+        self.H, self.P, self.N, self.G = heads, vdim, state, groups
+        self.K, self.norm_groups, self.eps = int(conv), norm_groups, float(eps)
+        self.inner = heads * vdim
+        self.conv_cols = self.inner + 2 * groups * state
+        self.in_cols = self.inner + self.conv_cols + heads
+        self.bias_cols = 0
+        self.conv = nn.Parameter(torch.zeros(self.conv_cols, self.K))
+        self.conv_b = nn.Parameter(torch.zeros(self.conv_cols))
+        self.dt_bias = nn.Parameter(torch.zeros(heads))
+        self.A_log = nn.Parameter(torch.zeros(heads))
+        self.D = nn.Parameter(torch.ones(heads))
+        self.norm = nn.Parameter(torch.ones(self.inner))
+        self.o_proj = TLLinear(self.inner, width, bias=False)
+        self.state_shapes = [(self.K - 1, self.conv_cols),
+                             (heads, state, vdim)]
+
+    def forward(self, proj, col, meta, hist, S):
+        inner, GN = self.inner, self.G * self.N
+        xbc = mx.conv_rope_rows(proj, col + inner, 1, self.conv_cols,
+                                self._f32("conv"), hist, meta,
+                                bias=self._f32("conv_b"), silu=True)
+        y = mx.ssd_scan(xbc, (0, inner, inner + GN), proj,
+                        col + inner + self.conv_cols, self._f32("dt_bias"),
+                        self._f32("A_log"), self._f32("D"), S, meta, self.H,
+                        self.P, self.N, self.G)
+        u = mx.gated_group_rms(y, proj, col, self._f32("norm"),
+                               self.norm_groups, self.eps,
+                               out_dtype=proj.dtype)
+        return self.o_proj(u)
+
+
+class ParallelMixer(nn.Module, _F32Cache):
+    """Two mixers side by side on the same input: ``left`` (attention) and
+    ``right`` (state-space), fed by ONE fused input projection. The result
+    is half the sum of the two outputs after each is RMS-normed over the
+    model width with its plain weight (``left_out`` / ``right_out``);
+    ``forward`` returns the two raw outputs and the caller's residual
+    update applies the norms and the half sum in the same pass."""
+
+    kind = "parallel"
+
+    def __init__(self, width: int, left: nn.Module, right: nn.Module):
+        super().__init__()
+        self.left, self.right = left, right
+        self.proj = TLLinear(width, left.in_cols + right.in_cols, bias=True)
+        self.left_out = nn.Parameter(torch.ones(width))
+        self.right_out = nn.Parameter(torch.ones(width))
+        self.state_shapes = list(left.state_shapes) + list(right.state_shapes)
+
+    def cache_spec(self):
+        return dict(self.left.cache_spec(), shapes=self.state_shapes)
+
+    def forward(self, h, meta, kpool, vpool, states):
+        proj = self.proj(h)
+        nl = len(self.left.state_shapes)
+        a = self.left(proj, 0, meta, kpool, vpool, *states[:nl])
+        b = self.right(proj, self.left.in_cols, meta, *states[nl:])
+        return a, b
+
+
+class PolyNormFF(nn.Module, _F32Cache):
+    """down(polynorm(up x)): the activation is a learned cubic in the
+    row-normalised powers of its input, coefficients ``act`` [4]."""
+
+    def __init__(self, width: int, ff: int, eps: float):
+        super().__init__()
+        self.eps = float(eps)
+        self.up = TLLinear(width, ff, bias=False)
+        self.down = TLLinear(ff, width, bias=False)
+        self.act = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0]))
+
+    def forward(self, h):
+        return self.down(mx.polynorm(self.up(h), self._f32("act"), self.eps))

@@ -155,7 +155,8 @@ class HybridSlotCache(DynamicPagedKVCache):
     state indexed by slot.
 
     ``specs[l]`` is ``{"kind": "kv", "G", "DK", "V"}`` (``V`` = 0: key
-    rows only, for layers whose values are part of the key row),
+    rows only, for layers whose values are part of the key row; an optional
+    ``"shapes"`` list adds fp32 per-slot state tensors beside the pools),
     ``{"kind": "kv_ref", "src": j}``, ``{"kind": "mlstm", "H", "D",
     "V"}`` or ``{"kind": "state", "shapes": [...]}``. ``k[l]`` / ``v[l]``
     are [pool_pages, G, PAGE, DK|V] (None for recurrent layers, the
@@ -180,7 +181,12 @@ class HybridSlotCache(DynamicPagedKVCache):
                 self.v.append(torch.zeros(pool_pages, sp["G"], PAGE,
                                           sp["V"], device=device,
                                           dtype=dtype) if sp["V"] else None)
-                self.state.append(None)
+                # a paged layer may keep fp32 per-slot state beside its
+                # pools (convolution histories, a parallel recurrence)
+                self.state.append(tuple(
+                    torch.zeros(slots, *shape, device=device,
+                                dtype=torch.float32)
+                    for shape in sp["shapes"]) if sp.get("shapes") else None)
             elif sp["kind"] == "kv_ref":
                 self.k.append(self.k[sp["src"]])
                 self.v.append(self.v[sp["src"]])

@@ -70,15 +70,19 @@ class RaggedMeta:
         first position): the step's tokens cut into per-sequence tiles for
         the tiled attention kernel."""
         if self._tiles is None:
+            self._tiles = {}
+        hit = self._tiles.get(size)
+        if hit is None:
             rows = []
             for b in range(self.B):
                 for o in range(0, self.new_h[b], size):
                     rows.append([b, self.cu_h[b] + o,
                                  min(size, self.new_h[b] - o),
                                  self.pos0_h[b] + o])
-            self._tiles = torch.tensor(rows, dtype=torch.int32).reshape(
+            hit = torch.tensor(rows, dtype=torch.int32).reshape(
                 -1, 4).to(self._device)
-        return self._tiles
+            self._tiles[size] = hit
+        return hit
 
     def scan_chunks(self, size: int):
         """The step's tokens cut into per-sequence chunks of ``size`` for
@@ -493,6 +497,8 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
                    vpool: Optional[torch.Tensor], meta: RaggedMeta, H: int,
                    scale: float, *, window: int = 0, sink: bool = False,
                    talk: Optional[torch.Tensor] = None, v_cols: int = 0,
+                   softcap: float = 0.0,
+                   sink_logits: Optional[torch.Tensor] = None,
                    out_dtype=torch.float32) -> torch.Tensor:
     """Causal attention of the step's tokens over their sequences' cached
     rows (the step's own rows already appended).
@@ -501,13 +507,20 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
     values from vpool [pages, G, PAGE, V], or, without it, the first
     ``v_cols`` columns of the key row. score = q.k * scale; with ``talk``
     [H, H] the heads' scores are mixed, s_h <- sum_g talk[h, g] s_g;
+    ``softcap`` > 0 replaces a score by softcap * tanh(score / softcap);
     ``window`` > 0 keeps keys with 0 <= i - j < window; ``sink`` adds one
-    to the softmax denominator. Scores, weights and sums are fp32.
+    to the softmax denominator, ``sink_logits`` [H] (fp32) adds
+    exp(sink_logits[h]) instead (a keyless, valueless entry that is neither
+    scaled nor capped). Scores, weights and sums are fp32.
     Returns [T, H*V] in ``out_dtype``."""
     G, DK = kpool.shape[1], kpool.shape[3]
     V = vpool.shape[3] if vpool is not None else v_cols
     T = q.shape[0]
     assert q.dtype == torch.float32 and q.shape[1] == H * DK
+    if sink_logits is not None:
+        assert sink_logits.dtype == torch.float32 \
+            and sink_logits.numel() == H
+        sink = True
     if q.is_cuda:
         if (kpool.dtype == torch.bfloat16 and meta.T > meta.B
                 and not os.environ.get("TL_NO_ATTN_TILES")
@@ -517,7 +530,7 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
             return _ext().flex_attn_tiles(
                 q, kpool, vpool, meta.query_tiles(), meta.table, talk,
                 int(H), float(scale), int(window), bool(sink), int(V),
-                out_dtype == torch.float32)
+                out_dtype == torch.float32, float(softcap), sink_logits)
         # few rows over long key ranges (decoding): spread each row's
         # keys over several blocks so the chip is filled; a function of
         # the step's shape only
@@ -530,7 +543,8 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
                                      meta.tok_pos, meta.table, talk, int(H),
                                      float(scale), int(window), bool(sink),
                                      int(V), out_dtype == torch.float32,
-                                     n_split, 1 if meta.T * H <= 512 else 8)
+                                     n_split, 1 if meta.T * H <= 512 else 8,
+                                     float(softcap), sink_logits)
     out = torch.empty(T, H, V)
     qf = q.view(T, H, DK)
     rep = H // G
@@ -548,6 +562,8 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
         sc = torch.einsum("thd,jhd->htj", qf[t0:t1], kb) * scale
         if talk is not None:
             sc = torch.einsum("hg,gtj->htj", talk.float(), sc)
+        if softcap:
+            sc = softcap * torch.tanh(sc / softcap)
         qpos = torch.arange(meta.pos0_h[b], L).view(-1, 1)
         kpos = torch.arange(L).view(1, -1)
         hide = kpos > qpos
@@ -556,11 +572,13 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
         sc = sc.masked_fill(hide, float("-inf"))
         m = sc.amax(-1, keepdim=True)
         if sink:
-            m = m.clamp_min(0.0)
+            sl = (sink_logits.view(H, 1, 1) if sink_logits is not None
+                  else torch.zeros(H, 1, 1))
+            m = torch.maximum(m, sl)
         e = torch.exp(sc - m)
         den = e.sum(-1, keepdim=True)
         if sink:
-            den = den + torch.exp(-m)
+            den = den + torch.exp(sl - m)
         out[t0:t1] = torch.einsum("htj,jhv->thv", e / den, vb)
     return out.reshape(T, H * V).to(out_dtype)
 
@@ -624,3 +642,257 @@ def lightning_scan(proj: torch.Tensor, offs, decay: torch.Tensor,
         if meta.new_h[b] > 0:
             S[slot] = Sb
     return o.reshape(T, H * V)
+
+
+# ---------------------------------------------------------------------------
+# layer norm with a weight and no bias, causal per-channel convolutions
+# whose last inputs live in the slot state, PolyNorm, grouped gated RMS,
+# the selective state-space recurrence
+# ---------------------------------------------------------------------------
+CONV_TILE = 8        # tokens per block of the convolution kernels
+
+
+def _ln(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    d = x - x.mean(-1, keepdim=True)
+    return d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w
+
+
+def _conv_ragged(u: torch.Tensor, w: torch.Tensor, hist: torch.Tensor,
+                 meta: RaggedMeta) -> torch.Tensor:
+    """Torch form of the causal convolution over a ragged step:
+    y_t = sum_j w[:, j] u_(t-K+1+j); inputs before a portion's start come
+    from hist[slot] (zeros for a sequence with no cached tokens), which is
+    left holding the sequence's last K-1 inputs."""
+    K = w.shape[1]
+    y = torch.empty_like(u)
+    for b in range(meta.B):
+        t0, t1 = meta.cu_h[b], meta.cu_h[b + 1]
+        if t1 == t0:
+            continue
+        slot = meta.slots_h[b]
+        prev = (torch.zeros(K - 1, u.shape[1]) if meta.pos0_h[b] == 0
+                else hist[slot].clone())
+        ext = torch.cat([prev, u[t0:t1]], 0)
+        n = t1 - t0
+        acc = torch.zeros(n, u.shape[1])
+        for j in range(K):
+            acc += w[:, j] * ext[j:j + n]
+        y[t0:t1] = acc
+        if K > 1:
+            hist[slot] = ext[ext.shape[0] - (K - 1):]
+    return y
+
+
+def layer_norm_rows(x: torch.Tensor, w: torch.Tensor, eps: float,
+                    out_dtype=torch.float32) -> torch.Tensor:
+    """(x - mean) / sqrt(var + eps) * w over the last axis of x [T, W]
+    (fp32; var = mean of squared deviations)."""
+    assert x.dtype == torch.float32 and w.dtype == torch.float32
+    if x.is_cuda:
+        return _ext().layer_norm_rows(x.contiguous(), w, float(eps),
+                                      out_dtype == torch.float32)
+    return _ln(x, w, eps).to(out_dtype)
+
+
+def ln_canon(X: torch.Tensor, w: torch.Tensor, eps: float,
+             conv_w: torch.Tensor, hist: torch.Tensor, meta: RaggedMeta,
+             out_dtype=torch.float32) -> torch.Tensor:
+    """A sublayer's input: h = layer_norm(X) * w, then h + conv(h) with the
+    causal per-channel taps conv_w [W, K]. hist [slots, K-1, W] (fp32)
+    holds every sequence's last K-1 normed rows and is updated; a sequence
+    with no cached tokens starts from zeros whatever its slot holds.
+    Everything in fp32; returns [T, W] in ``out_dtype``."""
+    assert X.dtype == torch.float32 and hist.dtype == torch.float32
+    K = conv_w.shape[1]
+    assert hist.shape[1] == K - 1 and K - 1 <= CONV_TILE
+    if X.is_cuda:
+        return _ext().ln_canon(X, w, float(eps), conv_w, hist,
+                               meta.query_tiles(CONV_TILE), meta.cu,
+                               meta.slots, meta.pos0,
+                               out_dtype == torch.float32)
+    h = _ln(X, w, eps)
+    return (h + _conv_ragged(h, conv_w, hist, meta)).to(out_dtype)
+
+
+def conv_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
+                   conv_w: torch.Tensor, hist: torch.Tensor,
+                   meta: RaggedMeta, *, bias: Optional[torch.Tensor] = None,
+                   silu: bool = False, rot_dims: int = 0,
+                   freqs: Optional[torch.Tensor] = None,
+                   rot_mult: float = 1.0,
+                   pool: Optional[torch.Tensor] = None,
+                   raw_pool: Optional[torch.Tensor] = None,
+                   pool_heads: int = 0):
+    """Short causal convolution over time on columns
+    [col, col + n_heads*head_dim) of src [T, L] (taps conv_w [N, K], fp32;
+    optional per-channel bias and silu), then rotate-half positions on the
+    first ``rot_dims`` dimensions of every head (angle pos * freqs[i], cos
+    and sin times ``rot_mult``). hist [slots, K-1, N] (fp32) holds every
+    sequence's last K-1 projected rows and is updated. The first
+    n_heads - pool_heads heads are returned densely as fp32
+    [T, (n_heads - pool_heads)*head_dim]; the last ``pool_heads`` heads
+    are scattered to the tokens' page rows of ``pool``
+    [pages, pool_heads, PAGE, head_dim] after rotation and, with
+    ``raw_pool``, as they leave the convolution (before rotation) too."""
+    N = n_heads * head_dim
+    T = src.shape[0]
+    K = conv_w.shape[1]
+    assert conv_w.shape[0] == N and hist.shape[1:] == (K - 1, N)
+    assert K - 1 <= CONV_TILE and rot_dims % 2 == 0 and rot_dims <= head_dim
+    assert (pool is None) == (pool_heads == 0) and pool_heads <= n_heads
+    dense = n_heads - pool_heads
+    if src.is_cuda:
+        out = torch.empty(T, dense * head_dim, device=src.device,
+                          dtype=torch.float32) if dense else None
+        _ext().conv_rope_rows(src, int(col), int(n_heads), int(head_dim),
+                              conv_w, bias, bool(silu), hist, int(rot_dims),
+                              freqs, float(rot_mult),
+                              meta.query_tiles(CONV_TILE), meta.cu,
+                              meta.slots, meta.pos0, meta.table, out, pool,
+                              raw_pool, int(pool_heads))
+        return out
+    y = _conv_ragged(src[:, col:col + N].float(), conv_w, hist, meta)
+    if bias is not None:
+        y = y + bias
+    if silu:
+        y = torch.nn.functional.silu(y)
+    raw = y.reshape(T, n_heads, head_dim)
+    x = raw.clone()
+    pos = meta.tok_pos.long()
+    if rot_dims:
+        half = rot_dims // 2
+        ang = pos.double().view(T, 1, 1) * freqs.double().view(1, 1, half)
+        c = (torch.cos(ang) * rot_mult).float()
+        s = (torch.sin(ang) * rot_mult).float()
+        u, v = raw[:, :, :half], raw[:, :, half:rot_dims]
+        x[:, :, :half] = u * c - v * s
+        x[:, :, half:rot_dims] = v * c + u * s
+    if pool is not None:
+        page = meta.table.long()[meta.tok_seq.long(), pos // PAGE]
+        pool[page, :, pos % PAGE] = x[:, dense:].to(pool.dtype)
+        if raw_pool is not None:
+            raw_pool[page, :, pos % PAGE] = raw[:, dense:].to(raw_pool.dtype)
+    return x[:, :dense].reshape(T, dense * head_dim) if dense else None
+
+
+def yarn_freqs(dims: int, base: float, scaling: Optional[dict], device):
+    """Rotation frequencies (float64 [dims/2]) and the multiplier of cos and
+    sin. Without ``scaling``: f_i = base^(-2i/dims), multiplier 1. With
+    ``scaling`` = {factor, original, fast, slow}: pairs that turn more than
+    ``fast`` times over ``original`` positions keep f_i, pairs that turn
+    fewer than ``slow`` times get f_i / factor, a linear ramp over the pair
+    index lies between; the multiplier is 0.1 ln(factor) + 1."""
+    f = rope_freqs(dims, base, "cpu")
+    if not scaling:
+        return f.to(device), 1.0
+    import math
+    factor = float(scaling["factor"])
+
+    def pair_of(turns):
+        return dims * math.log(scaling["original"]
+                               / (2.0 * math.pi * turns)) / (
+                                   2.0 * math.log(base))
+
+    lo = max(math.floor(pair_of(scaling["fast"])), 0)
+    hi = min(math.ceil(pair_of(scaling["slow"])), dims - 1)
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.to(device), 0.1 * math.log(factor) + 1.0
+
+
+def ssd_scan(xbc: torch.Tensor, offs, dt_src: torch.Tensor, dt_col: int,
+             dt_bias: torch.Tensor, A_log: torch.Tensor, skip: torch.Tensor,
+             S: torch.Tensor, meta: RaggedMeta, H: int, P: int, N: int,
+             G: int) -> torch.Tensor:
+    """Selective state-space recurrence with one scalar decay per head and
+    token. xbc [T, *] (fp32) holds x [H*P] | B [G*N] | C [G*N] at columns
+    ``offs``; the raw step sizes are columns [dt_col, dt_col + H) of
+    dt_src. Per head h (group floor(h / (H/G))):
+
+        dt = softplus(raw + dt_bias_h)
+        S_t = exp(-exp(A_log_h) dt) S_(t-1) + dt B_t x_t^T     (S is [N, P])
+        y_t = S_t^T C_t + skip_h x_t
+
+    The state pool S [slots, H, N, P] (fp32) is read at ``meta.slots``
+    (zeros for a sequence with no cached tokens) and written back. All in
+    fp32; returns y [T, H*P] fp32."""
+    x_off, b_off, c_off = offs
+    T = xbc.shape[0]
+    assert xbc.dtype == torch.float32 and S.dtype == torch.float32
+    assert S.shape[1:] == (H, N, P) and H % G == 0
+    if xbc.is_cuda:
+        return _ext().ssd_scan(xbc, int(x_off), int(b_off), int(c_off),
+                               dt_src, int(dt_col), dt_bias, A_log, skip, S,
+                               meta.cu, meta.slots, meta.pos0, int(H),
+                               int(P), int(N), int(G))
+    x = xbc[:, x_off:x_off + H * P].view(T, H, P)
+    rep = H // G
+    Bm = xbc[:, b_off:b_off + G * N].view(T, G, N).repeat_interleave(rep, 1)
+    Cm = xbc[:, c_off:c_off + G * N].view(T, G, N).repeat_interleave(rep, 1)
+    dt = torch.nn.functional.softplus(
+        dt_src[:, dt_col:dt_col + H].float() + dt_bias)
+    dec = torch.exp(-torch.exp(A_log) * dt)                    # [T, H]
+    y = torch.empty(T, H, P)
+    for b in range(meta.B):
+        t0, t1 = meta.cu_h[b], meta.cu_h[b + 1]
+        if t1 == t0:
+            continue
+        slot = meta.slots_h[b]
+        Sb = (torch.zeros(H, N, P) if meta.pos0_h[b] == 0
+              else S[slot].clone())
+        for t in range(t0, t1):
+            Sb = dec[t].view(H, 1, 1) * Sb + (dt[t].view(H, 1) * Bm[t]
+                                              ).unsqueeze(-1) * x[t].unsqueeze(1)
+            y[t] = (Sb * Cm[t].unsqueeze(-1)).sum(1) + skip.view(H, 1) * x[t]
+        S[slot] = Sb
+    return y.reshape(T, H * P)
+
+
+def gated_group_rms(y: torch.Tensor, gate: torch.Tensor, gate_col: int,
+                    w: torch.Tensor, groups: int, eps: float,
+                    out_dtype=torch.float32) -> torch.Tensor:
+    """u = y * silu(gate[:, gate_col:gate_col + N]); every one of
+    ``groups`` equal parts of a row of u is divided by its own root mean
+    square; times w [N]. y [T, N] fp32; fp32 arithmetic."""
+    N = y.shape[1]
+    assert y.dtype == torch.float32 and N % groups == 0
+    if y.is_cuda:
+        return _ext().gated_group_rms(y.contiguous(), gate, int(gate_col), w,
+                                      int(groups), float(eps),
+                                      out_dtype == torch.float32)
+    u = y * torch.nn.functional.silu(gate[:, gate_col:gate_col + N].float())
+    u = _rms(u.view(-1, groups, N // groups), eps).reshape(-1, N)
+    return (u * w).to(out_dtype)
+
+
+def postln_add(X: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float,
+               y2: Optional[torch.Tensor] = None,
+               wy: Optional[torch.Tensor] = None,
+               wy2: Optional[torch.Tensor] = None) -> None:
+    """Residual with a layer norm on the sublayer's OUTPUT, in place on the
+    fp32 residual X [T, W]:  X += layer_norm(u) * w.  u = y, or with two
+    branch outputs u = (y / rms(y) * wy + y2 / rms(y2) * wy2) / 2."""
+    assert X.dtype == torch.float32 and w.dtype == torch.float32
+    if X.is_cuda:
+        _ext().postln_add(X, y.contiguous(), w, float(eps),
+                          None if y2 is None else y2.contiguous(), wy, wy2)
+        return
+    u = y.float()
+    if y2 is not None:
+        u = 0.5 * (_rms(u, eps) * wy + _rms(y2.float(), eps) * wy2)
+    X += _ln(u, w, eps)
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3] with
+    element-wise powers and N(u) = u / rms(u) over a row; fp32 arithmetic,
+    result in z's dtype."""
+    assert coef.dtype == torch.float32 and coef.numel() == 4
+    if z.is_cuda:
+        return _ext().polynorm(z.contiguous(), coef, float(eps))
+    f = z.float()
+    f2 = f * f
+    out = (coef[0] * _rms(f, eps) + coef[1] * _rms(f2, eps)
+           + coef[2] * _rms(f2 * f, eps) + coef[3])
+    return out.to(z.dtype)
