@@ -492,10 +492,12 @@ Tensor moe_gemm(Tensor x, c10::optional<Tensor> tok_idx, Tensor seg_off,
 
 void register_mix_ops(pybind11::module& mod);  // bindings_mix.cpp
 void register_seq_ops(pybind11::module& mod);  // bindings_seq.cpp
+void register_ssm_ops(pybind11::module& mod);  // bindings_ssm.cpp
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
   register_mix_ops(mod);
   register_seq_ops(mod);
+  register_ssm_ops(mod);
   mod.def("rope_append_", &rope_append_,
           "fused RoPE + KV-cache append from fused-QKV rows");
   mod.def("swiglu_fused", &swiglu_fused, "silu-mul on fused [.,2I] rows");

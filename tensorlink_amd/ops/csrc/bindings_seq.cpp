@@ -32,7 +32,8 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       const void* table, int P, const void* talk, void* out,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
-                      int pool_f32, int hb_max, hipStream_t stream);
+                      int pool_f32, int hb_max, float softcap,
+                      const void* sinks, hipStream_t stream);
 int tl_flex_attn_tiles_ok(int H, int G, int KG, int DK, int V);
 void tl_stage_queries(const void* q, const void* talk, void* out, int T,
                       int H, int G, int DK, hipStream_t stream);
@@ -40,7 +41,8 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                        int vld, const void* tiles, int n_tiles,
                        const void* table, int P, void* out, int out_f32,
                        int H, int G, int KG, int DK, int V, float scale,
-                       int window, int sink, hipStream_t stream);
+                       int window, int sink, float softcap, const void* sinks,
+                       hipStream_t stream);
 int tl_lightning_scan(const void* proj, int ld, int q_off, int k_off,
                       int v_off, const void* decay, void* S, const void* cu,
                       const void* slots, const void* pos0, void* out, int B,
@@ -221,7 +223,12 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
                       Tensor tok_seq, Tensor tok_pos, Tensor table,
                       c10::optional<Tensor> talk, int64_t H, double scale,
                       int64_t window, bool sink, int64_t V, bool out_f32,
-                      int64_t n_split, int64_t hb_max) {
+                      int64_t n_split, int64_t hb_max, double softcap,
+                      c10::optional<Tensor> sinks) {
+  if (sinks.has_value()) {
+    SEQ_F32(sinks.value());
+    TORCH_CHECK(sinks->numel() == H && sink, "sink logits must be [H]");
+  }
   SEQ_F32(q);
   SEQ_IN(kpool);
   SEQ_I32(tok_seq);
@@ -273,7 +280,8 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
       talk.has_value() ? talk->data_ptr() : nullptr, out.data_ptr(),
       out_f32 ? 1 : 0, n_split > 1 ? part.data_ptr() : nullptr, (int)n_split,
       (int)T, (int)H, G, DK, (int)V, (float)scale, (int)window, sink ? 1 : 0,
-      pool_f32, (int)std::max<int64_t>(1, hb_max), seq_stream());
+      pool_f32, (int)std::max<int64_t>(1, hb_max), (float)softcap,
+      sinks.has_value() ? sinks->data_ptr() : nullptr, seq_stream());
   TORCH_CHECK(rc == 0, "flex_attn_rows: launch refused");
   return out;
 }
@@ -289,7 +297,12 @@ bool flex_attn_tiles_ok(int64_t H, int64_t G, bool has_talk, int64_t DK,
 Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
                        Tensor tiles, Tensor table,
                        c10::optional<Tensor> talk, int64_t H, double scale,
-                       int64_t window, bool sink, int64_t V, bool out_f32) {
+                       int64_t window, bool sink, int64_t V, bool out_f32,
+                       double softcap, c10::optional<Tensor> sinks) {
+  if (sinks.has_value()) {
+    SEQ_F32(sinks.value());
+    TORCH_CHECK(sinks->numel() == H && sink, "sink logits must be [H]");
+  }
   SEQ_F32(q);
   SEQ_IN(kpool);
   SEQ_I32(tiles);
@@ -337,7 +350,8 @@ Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
       qs.data_ptr(), kpool.data_ptr(), vp, vld, tiles.data_ptr(),
       (int)tiles.size(0), table.data_ptr(), (int)table.size(1),
       out.data_ptr(), out_f32 ? 1 : 0, (int)H, G, KG, DK, (int)V,
-      (float)scale, (int)window, sink ? 1 : 0, seq_stream());
+      (float)scale, (int)window, sink ? 1 : 0, (float)softcap,
+      sinks.has_value() ? sinks->data_ptr() : nullptr, seq_stream());
   TORCH_CHECK(rc == 0, "flex_attn_tiles: launch refused");
   return out;
 }

@@ -101,7 +101,7 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
     const int* __restrict__ tok_pos, const int* __restrict__ table, int P,
     const float* __restrict__ talk, void* __restrict__ out, int out_f32,
     float* __restrict__ part, int H, int G, int DK, int V, float scale,
-    int window, int sink) {
+    int window, int sink, float softcap, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   const int t = blockIdx.x, h0 = blockIdx.y * HB;
   const int ns = gridDim.z, z = blockIdx.z;
@@ -182,7 +182,8 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
     float p[HB];
 #pragma unroll
     for (int b = 0; b < HB; ++b) {
-      const float sv = valid ? s[b] : -INFINITY;
+      const float sc = softcap > 0.f ? softcap * tanhf(s[b] / softcap) : s[b];
+      const float sv = valid ? sc : -INFINITY;
       const float nm = fmaxf(m[b], wave_reduce_max(sv));
       // nm is finite: every tile of the loop holds at least one valid key
       const float c = expf(m[b] - nm);
@@ -257,13 +258,14 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       }
       continue;
     }
-    if (sink) M = fmaxf(M, 0.f);
+    const float sl = sinks ? sinks[h0 + b] : 0.f;   // the sink's logit
+    if (sink) M = fmaxf(M, sl);
     for (int w = 0; w < NWAVE; ++w) {
       const float mw = stat[(w * HB + b) * 2];
       f[w] = (mw == -INFINITY) ? 0.f : expf(mw - M);
       L += f[w] * stat[(w * HB + b) * 2 + 1];
     }
-    if (sink) L += expf(-M);
+    if (sink) L += expf(sl - M);
     for (int c = threadIdx.x; c < V; c += BLOCK) {
       float A = 0.f;
       for (int w = 0; w < NWAVE; ++w) A += f[w] * accs[(w * HB + b) * V + c];
@@ -279,13 +281,14 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
 // one block per (token, head): merge the key splits
 __global__ __launch_bounds__(BLOCK) void flex_attn_merge_kernel(
     const float* __restrict__ part, void* __restrict__ out, int out_f32,
-    int ns, int V, int sink) {
+    int ns, int V, int sink, int H, const float* __restrict__ sinks) {
   const int64_t row = blockIdx.x;
   const float* pr = part + row * ns * (2 + V);
   float M = -INFINITY;
   for (int z = 0; z < ns; ++z) M = fmaxf(M, pr[z * (2 + V)]);
-  if (sink) M = fmaxf(M, 0.f);
-  float L = sink ? expf(-M) : 0.f;
+  const float sl = sinks ? sinks[row % H] : 0.f;
+  if (sink) M = fmaxf(M, sl);
+  float L = sink ? expf(sl - M) : 0.f;
   for (int z = 0; z < ns; ++z) {
     const float mz = pr[z * (2 + V)];
     L += (mz == -INFINITY ? 0.f : expf(mz - M)) * pr[z * (2 + V) + 1];
@@ -309,17 +312,17 @@ void launch_rows(bool has_talk, dim3 grid, size_t smem, hipStream_t stream,
                  const int* tok_seq, const int* tok_pos, const int* table,
                  int P, const float* talk, void* out, int out_f32,
                  float* part, int H, int G, int DK, int V, float scale,
-                 int window, int sink) {
+                 int window, int sink, float softcap, const float* sinks) {
   if (has_talk)
     hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, true>), grid,
                        dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
                        tok_seq, tok_pos, table, P, talk, out, out_f32, part,
-                       H, G, DK, V, scale, window, sink);
+                       H, G, DK, V, scale, window, sink, softcap, sinks);
   else
     hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, false>), grid,
                        dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
                        tok_seq, tok_pos, table, P, talk, out, out_f32, part,
-                       H, G, DK, V, scale, window, sink);
+                       H, G, DK, V, scale, window, sink, softcap, sinks);
 }
 
 size_t rows_smem(bool has_talk, int hb, int G, int DK, int V) {
@@ -383,7 +386,8 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       const void* table, int P, const void* talk, void* out,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
-                      int pool_f32, int hb_max, hipStream_t stream) {
+                      int pool_f32, int hb_max, float softcap,
+                      const void* sinks, hipStream_t stream) {
   if (T <= 0) return 0;
   const bool has_talk = talk != nullptr;
   const int hb = heads_per_block(H, G, DK, V, has_talk ? 1 : 0, hb_max);
@@ -397,7 +401,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                             (const int*)tok_seq, (const int*)tok_pos,        \
                             (const int*)table, P, (const float*)talk, out,   \
                             out_f32, (float*)part, H, G, DK, V, scale,       \
-                            window, sink)
+                            window, sink, softcap, (const float*)sinks)
 #define TL_FA_V(TT, HBB)                     \
   if (vr <= 1) TL_FA(TT, HBB, 1);            \
   else if (vr <= 2) TL_FA(TT, HBB, 2);       \
@@ -418,7 +422,8 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
 #undef TL_FA
   if (ns > 1)
     hipLaunchKernelGGL(flex_attn_merge_kernel, dim3(T * H), dim3(BLOCK), 0,
-                       stream, (const float*)part, out, out_f32, ns, V, sink);
+                       stream, (const float*)part, out, out_f32, ns, V, sink, H,
+                       (const float*)sinks);
   return 0;
 }
 

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
     const int* __restrict__ tiles,   // [n][4]: seq, first token, count, pos
     const int* __restrict__ table, int P, void* __restrict__ out,
     int out_f32, int H, int G, int KG, int DK, int V, float scale,
-    int window, int sink) {
+    int window, int sink, float softcap, const float* __restrict__ sinks) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16* vt_lds = reinterpret_cast<bf16*>(smem_raw);     // [V][VLD]
 
@@ -189,7 +189,9 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
           const int key = kb + t16 * 16 + quad * 4 + r;
           const bool ok =
               key <= qpos && (window <= 0 || key > qpos - window);
-          const float s = ok ? st[t16][r] * scale : -INFINITY;
+          float s = st[t16][r] * scale;
+          if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+          s = ok ? s : -INFINITY;
           sv[t16 * 4 + r] = s;
           mx = fmaxf(mx, s);
         }
@@ -238,9 +240,10 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
   // every query sees itself, so mrun is finite here
   float f = 1.f;
   if (sink) {
-    const float m_fin = fmaxf(mrun, 0.f);
+    const float sl = sinks ? sinks[h] : 0.f;      // the sink's logit
+    const float m_fin = fmaxf(mrun, sl);
     f = __expf(mrun - m_fin);
-    l = l * f + __expf(-m_fin);
+    l = l * f + __expf(sl - m_fin);
   }
   const float inv = f / l;
   if (q_valid) {
@@ -288,7 +291,8 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                        int vld, const void* tiles, int n_tiles,
                        const void* table, int P, void* out, int out_f32,
                        int H, int G, int KG, int DK, int V, float scale,
-                       int window, int sink, hipStream_t stream) {
+                       int window, int sink, float softcap, const void* sinks,
+                       hipStream_t stream) {
   if (!tl_flex_attn_tiles_ok(H, G, KG, DK, V) || vld % 8 != 0 ||
       n_tiles <= 0)
     return 1;
@@ -300,7 +304,7 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                      stream, (const bf16*)q, (const bf16*)kpool,             \
                      (const bf16*)vpool, vld, (const int*)tiles,             \
                      (const int*)table, P, out, out_f32, H, G, KG, DK, V,    \
-                     scale, window, sink)
+                     scale, window, sink, softcap, (const float*)sinks)
 #define TL_FT_V(QCC)                          \
   if (nvt <= 4) TL_FT_LAUNCH(QCC, 4);         \
   else if (nvt <= 8) TL_FT_LAUNCH(QCC, 8);    \
