@@ -167,15 +167,14 @@ def polynorm_ff(h, W, pre, eps):
 
 def layer(x, W, i, lc, cfg):
     eps = cfg["norm"]["eps"]
-    taps_w1, taps_w2 = W[f"l{i}.canon1"], W[f"l{i}.canon2"]
     h = layer_norm(x, W[f"l{i}.norm1"], eps)
-    h = h + causal_conv(h, taps_w1)
+    h = h + causal_conv(h, W[f"l{i}.canon1"])
     assert lc["type"] == "parallel"
     y = parallel_mixer(h, W, f"l{i}.mix.", lc["mixer"], eps)
     x = x + layer_norm(y, W[f"l{i}.norm1b"], eps)
     if lc.get("mlp") is not None:
         h = layer_norm(x, W[f"l{i}.norm2"], eps)
-        h = h + causal_conv(h, taps_w2)
+        h = h + causal_conv(h, W[f"l{i}.canon2"])
         y = polynorm_ff(h, W, f"l{i}.mlp.", eps)
         x = x + layer_norm(y, W[f"l{i}.norm2b"], eps)
     return x
