@@ -49,10 +49,11 @@ def parse_args():
                         "beside an equal-size Qwen3-MoE-shaped model")
     p.add_argument("--sizes", default="w1024,w2048",
                    help="layered mode: comma list of size presets")
-    p.add_argument("--family", choices=["kepusun", "senulix"],
+    p.add_argument("--family", choices=["kepusun", "senulix", "dizepel"],
                    default="kepusun",
                    help="layered mode: which layered family to time "
-                        "(senulix: beside an equal-size dense GQA decoder)")
+                        "(senulix, dizepel: beside an equal-size dense GQA "
+                        "decoder)")
     p.add_argument("--dp", type=int, default=1,
                    help="data-parallel replicas (train mode; world=dp*pp)")
     return p.parse_args()
@@ -203,6 +204,56 @@ def senulix_configs(z):
     return sen, ref
 
 
+DIZEPEL_SIZES = {
+    # six layers, the third and fourth run twice: eight layer runs
+    "w1024": dict(width=1024, heads=8, kv=2, dim=128, rot=64, ssm_heads=16,
+                  ssm_dim=64, state=128, groups=2, ff=4096, vocab=32000,
+                  batch=8, prompt=2048),
+    "w2048": dict(width=2048, heads=16, kv=4, dim=128, rot=64, ssm_heads=32,
+                  ssm_dim=64, state=128, groups=4, ff=8192, vocab=32000,
+                  batch=8, prompt=2048),
+    "tiny": dict(width=128, heads=2, kv=1, dim=32, rot=16, ssm_heads=4,
+                 ssm_dim=16, state=16, groups=1, ff=256, vocab=512, batch=2,
+                 prompt=96),
+}
+
+
+def dizepel_configs(z):
+    """(Dizepel config, dense GQA decoder) of a preset: same width,
+    vocabulary, attention heads and head size; the dense model has as many
+    layers as the Dizepel model has layer RUNS (equal depth of compute) and
+    its gated three-matrix feed-forward gets 2/3 of the two-matrix one's
+    width."""
+    from tensorlink_amd.models.configs import ModelConfig
+    from tensorlink_amd.models.dizepel import DizepelConfig
+    mixer = {
+        "left": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"],
+                 "vdim": z["dim"], "conv": 4, "scale": z["dim"] ** -0.5,
+                 "softcap": 50.0,
+                 "rot": {"dims": z["rot"], "base": 250000.0,
+                         "scaling": {"factor": 4.0, "original": 2048,
+                                     "fast": 32.0, "slow": 1.0}}},
+        "right": {"heads": z["ssm_heads"], "vdim": z["ssm_dim"],
+                  "state": z["state"], "groups": z["groups"], "conv": 4,
+                  "norm_groups": z["groups"]}}
+    layer = {"type": "parallel", "mixer": mixer,
+             "mlp": {"kind": "dense", "ff": z["ff"]}}
+    diz = DizepelConfig.from_dict({
+        "architecture": "Dizepel", "vocab": z["vocab"], "width": z["width"],
+        "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+        "canon": {"taps": 3}, "loop": {"start": 2, "stop": 4, "times": 2},
+        "layers": [layer] * 6}, name="dizepel-" + str(z["width"]))
+    ref = ModelConfig(
+        name="dense-gqa-" + str(z["width"]), vocab_size=z["vocab"],
+        hidden_size=z["width"],
+        intermediate_size=(2 * z["ff"] // 3 + 63) // 64 * 64,
+        num_hidden_layers=len(diz.layer_runs()),
+        num_attention_heads=z["heads"], num_key_value_heads=z["kv"],
+        head_dim=z["dim"], max_position_embeddings=8192,
+        architecture="qwen3")
+    return diz, ref
+
+
 @torch.no_grad()
 def run_layered(args, device, use_gpu):
     """Prefill and decode tokens/s of the Kepusun family beside the
@@ -252,7 +303,13 @@ def run_layered(args, device, use_gpu):
         return out
 
     for name in args.sizes.split(","):
-        if args.family == "senulix":
+        if args.family == "dizepel":
+            z = DIZEPEL_SIZES[name]
+            diz, ref = dizepel_configs(z)
+            B, S = z["batch"], z["prompt"]
+            res = {"dizepel": measure(diz, B, S),
+                   "dense_gqa": measure(ref, B, S)}
+        elif args.family == "senulix":
             z = SENULIX_SIZES[name]
             sen, ref = senulix_configs(z)
             B, S = z["batch"], z["prompt"]

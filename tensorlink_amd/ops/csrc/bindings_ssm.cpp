@@ -39,6 +39,18 @@ int tl_ssd_scan(const void* xbc, int ldx, int x_off, int b_off, int c_off,
                 const void* A_log, const void* skip, void* S, const void* cu,
                 const void* slots, const void* pos0, void* out, int B, int H,
                 int G, int N, int P, int dt_f32, hipStream_t stream);
+void tl_ssd_chunk_prep(const void* xbc, int ldx, int x_off, int b_off,
+                       int c_off, const void* dt_src, int ldd, int dt_col,
+                       const void* dt_bias, const void* A_log,
+                       const void* cu_c, void* Cs, void* Cd, void* Bs,
+                       void* Bw, void* Xd, void* Lc, void* tot, int NC, int H,
+                       int G, int N, int P, int C, int dt_f32,
+                       hipStream_t stream);
+void tl_ssd_decay_mask(void* A, const void* Lc, int NCH, int C,
+                       hipStream_t stream);
+void tl_ssd_chain(void* U, void* S, const void* tot, const void* chunk_base,
+                  const void* n_chunks, const void* slots, const void* pos0,
+                  int B, int H, int NP, hipStream_t stream);
 }
 
 namespace {
@@ -281,6 +293,79 @@ Tensor ssd_scan(Tensor xbc, int64_t x_off, int64_t b_off, int64_t c_off,
   return out;
 }
 
+// per-(chunk, head) operands of the chunk form:
+// Cs, Cd, Bs, Bw [chunks*H, C, N], Xd [chunks*H, C, P], L [chunks*H, C],
+// tot [chunks*H]
+std::vector<Tensor> ssd_chunk_prep(Tensor xbc, int64_t x_off, int64_t b_off,
+                                   int64_t c_off, Tensor dt_src,
+                                   int64_t dt_col, Tensor dt_bias,
+                                   Tensor A_log, Tensor cu_c, int64_t H,
+                                   int64_t P, int64_t N, int64_t G,
+                                   int64_t C) {
+  SSM_F32(xbc);
+  SSM_IN(dt_src);
+  SSM_F32(dt_bias);
+  SSM_F32(A_log);
+  SSM_I32(cu_c);
+  const int64_t L = xbc.size(1), NC = cu_c.numel() - 1;
+  TORCH_CHECK(xbc.dim() == 2 && dt_src.dim() == 2 &&
+                  dt_src.size(0) == xbc.size(0) && NC >= 0 && C >= 1,
+              "xbc [T, L], dt_src [T, *]");
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && x_off >= 0 &&
+                  x_off + H * P <= L && b_off >= 0 && b_off + G * N <= L &&
+                  c_off >= 0 && c_off + G * N <= L && dt_col >= 0 &&
+                  dt_col + H <= dt_src.size(1) && dt_bias.numel() == H &&
+                  A_log.numel() == H,
+              "columns out of range");
+  auto o = xbc.options();
+  std::vector<Tensor> r;
+  for (int i = 0; i < 4; ++i) r.push_back(torch::empty({NC * H, C, N}, o));
+  r.push_back(torch::empty({NC * H, C, P}, o));
+  r.push_back(torch::empty({NC * H, C}, o));
+  r.push_back(torch::empty({NC * H}, o));
+  tl_ssd_chunk_prep(xbc.data_ptr(), (int)L, (int)x_off, (int)b_off,
+                    (int)c_off, dt_src.data_ptr(), (int)dt_src.size(1),
+                    (int)dt_col, dt_bias.data_ptr(), A_log.data_ptr(),
+                    cu_c.data_ptr(), r[0].data_ptr(), r[1].data_ptr(),
+                    r[2].data_ptr(), r[3].data_ptr(), r[4].data_ptr(),
+                    r[5].data_ptr(), r[6].data_ptr(), (int)NC, (int)H, (int)G,
+                    (int)N, (int)P, (int)C, ssm_is_f32(dt_src), ssm_stream());
+  return r;
+}
+
+void ssd_decay_mask_(Tensor A, Tensor Lc) {
+  SSM_F32(A);
+  SSM_F32(Lc);
+  TORCH_CHECK(A.dim() == 3 && A.size(1) == A.size(2) && Lc.dim() == 2 &&
+                  Lc.size(0) == A.size(0) && Lc.size(1) == A.size(1),
+              "A must be [chunks*H, C, C], L [chunks*H, C]");
+  tl_ssd_decay_mask(A.data_ptr(), Lc.data_ptr(), (int)A.size(0),
+                    (int)A.size(1), ssm_stream());
+}
+
+void ssd_chain_(Tensor U, Tensor S, Tensor tot, Tensor chunk_base,
+                Tensor n_chunks, Tensor slots, Tensor pos0) {
+  SSM_F32(U);
+  SSM_F32(S);
+  SSM_F32(tot);
+  SSM_I32(chunk_base);
+  SSM_I32(n_chunks);
+  SSM_I32(slots);
+  SSM_I32(pos0);
+  TORCH_CHECK(S.dim() == 4, "S pool [slots, H, N, P]");
+  const int H = S.size(1);
+  const int64_t NP = S.size(2) * S.size(3);
+  TORCH_CHECK(tot.numel() % H == 0 && U.numel() == tot.numel() * NP,
+              "U must be [chunks*H, N, P], tot [chunks*H]");
+  const int B = slots.size(0);
+  TORCH_CHECK(chunk_base.size(0) == B && n_chunks.size(0) == B &&
+                  pos0.size(0) == B,
+              "per-sequence chunk metadata");
+  tl_ssd_chain(U.data_ptr(), S.data_ptr(), tot.data_ptr(),
+               chunk_base.data_ptr(), n_chunks.data_ptr(), slots.data_ptr(),
+               pos0.data_ptr(), B, H, (int)NP, ssm_stream());
+}
+
 }  // namespace
 
 void register_ssm_ops(pybind11::module& mod) {
@@ -297,6 +382,12 @@ void register_ssm_ops(pybind11::module& mod) {
   mod.def("conv_rope_rows", &conv_rope_rows,
           "short causal convolution + rotate-half positions, dense or "
           "scattered into page pools");
+  mod.def("ssd_chunk_prep", &ssd_chunk_prep,
+          "per-chunk operands of the chunk form of the state-space scan");
+  mod.def("ssd_decay_mask_", &ssd_decay_mask_,
+          "A[i][j] *= exp(L_i - L_j) below and on the diagonal, 0 above");
+  mod.def("ssd_chain_", &ssd_chain_,
+          "chunk summaries -> state before each chunk; final state to slot");
   mod.def("ssd_scan", &ssd_scan,
           "selective state-space scan over ragged sequences (slot state)");
 }

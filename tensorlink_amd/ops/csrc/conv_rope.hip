@@ -75,35 +75,52 @@ __global__ __launch_bounds__(BLOCK) void conv_rope_rows_kernel(
     const bool pair = r < half;
     const int d0 = pair ? r : r + half;
     const int ch0 = hd * D + d0, ch1 = ch0 + half;
-    float w0[MAXK], w1[MAXK];
+    // taps and the sliding window are aligned at the END of fixed-size
+    // arrays (leading entries zero), so every index is static
+    float w0[MAXK], w1[MAXK], u0[MAXK - 1], u1[MAXK - 1];
 #pragma unroll
-    for (int j = 0; j < MAXK; ++j) {
-      w0[j] = j < K ? taps[(int64_t)ch0 * K + j] : 0.f;
-      w1[j] = (pair && j < K) ? taps[(int64_t)ch1 * K + j] : 0.f;
+    for (int m = 0; m < MAXK; ++m) {
+      const int j = m - (MAXK - K);
+      w0[m] = j >= 0 ? taps[(int64_t)ch0 * K + j] : 0.f;
+      w1[m] = (pair && j >= 0) ? taps[(int64_t)ch1 * K + j] : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < MAXK - 1; ++m) {
+      const int j = m - (MAXK - K);
+      float a = 0.f, b = 0.f;
+      if (j >= 0) {
+        const int row = tok0 - (K - 1) + j;
+        if (row >= c0) {
+          a = ldf<T>(src, (int64_t)row * ld + col + ch0);
+          if (pair) b = ldf<T>(src, (int64_t)row * ld + col + ch1);
+        } else if (!fresh) {
+          const int64_t hr = (int64_t)(K - 1 + row - c0) * N;
+          a = hs[hr + ch0];
+          if (pair) b = hs[hr + ch1];
+        }
+      }
+      u0[m] = a;
+      u1[m] = b;
     }
     const float b0 = bias ? bias[ch0] : 0.f;
     const float b1 = (bias && pair) ? bias[ch1] : 0.f;
     for (int i = 0; i < n; ++i) {
-      float a0 = b0, a1 = b1;
+      const int64_t ro = (int64_t)(tok0 + i) * ld + col;
+      const float c0v = ldf<T>(src, ro + ch0);
+      const float c1v = pair ? ldf<T>(src, ro + ch1) : 0.f;
+      float a0 = b0 + w0[MAXK - 1] * c0v, a1 = b1 + w1[MAXK - 1] * c1v;
 #pragma unroll
-      for (int j = 0; j < MAXK; ++j) {
-        if (j < K) {
-          const int row = tok0 + i - (K - 1) + j;
-          float u0, u1 = 0.f;
-          if (row >= c0) {
-            u0 = ldf<T>(src, (int64_t)row * ld + col + ch0);
-            if (pair) u1 = ldf<T>(src, (int64_t)row * ld + col + ch1);
-          } else if (!fresh) {
-            const int64_t hr = (int64_t)(K - 1 + row - c0) * N;
-            u0 = hs[hr + ch0];
-            if (pair) u1 = hs[hr + ch1];
-          } else {
-            u0 = 0.f;
-          }
-          a0 += w0[j] * u0;
-          a1 += w1[j] * u1;
-        }
+      for (int m = 0; m < MAXK - 1; ++m) {
+        a0 += w0[m] * u0[m];
+        a1 += w1[m] * u1[m];
       }
+#pragma unroll
+      for (int m = 0; m < MAXK - 2; ++m) {
+        u0[m] = u0[m + 1];
+        u1[m] = u1[m + 1];
+      }
+      u0[MAXK - 2] = c0v;
+      u1[MAXK - 2] = c1v;
       if (act_silu) {
         a0 = silu_f(a0);
         a1 = silu_f(a1);

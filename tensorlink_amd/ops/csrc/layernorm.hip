@@ -37,6 +37,7 @@ constexpr int BLOCK = 256;
 constexpr int NW = BLOCK / WAVE_SIZE;
 constexpr int TILE = 8;           // tokens per block of tl_ln_canon
 constexpr int MAXROWS = 3 * TILE; // halo + tile + the portion's last rows
+constexpr int MAXK = TILE + 1;    // most taps (history of at most TILE rows)
 
 template <typename T> DEVINLINE float ldf(const T* p, int64_t i);
 template <> DEVINLINE float ldf<float>(const float* p, int64_t i) { return p[i]; }
@@ -117,22 +118,40 @@ __global__ __launch_bounds__(BLOCK) void ln_canon_kernel(
   float* hs = hist + (int64_t)slots[seq] * (K - 1) * W;
   for (int c = threadIdx.x; c < W; c += BLOCK) {
     const float wc = w[c];
-    const float* tc = taps + (int64_t)c * K;
-    for (int i = 0; i < n; ++i) {
-      float acc = 0.f, self = 0.f;
-      for (int j = 0; j < K; ++j) {
-        const int row = tok0 + i - (K - 1) + j;
-        float hv;
+    // taps and the sliding window of normed values are aligned at the END
+    // of fixed-size arrays (leading entries zero): every index is static
+    float tw[MAXK], hv[MAXK - 1];
+#pragma unroll
+    for (int m = 0; m < MAXK; ++m) {
+      const int j = m - (MAXK - K);
+      tw[m] = j >= 0 ? taps[(int64_t)c * K + j] : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < MAXK - 1; ++m) {
+      const int j = m - (MAXK - K);
+      float v = 0.f;
+      if (j >= 0) {
+        const int row = tok0 - (K - 1) + j;
         if (row >= c0) {
           const int si = row - r_lo;
-          hv = (X[(int64_t)row * W + c] - s_mean[si]) * s_rstd[si] * wc;
-        } else {
-          hv = fresh ? 0.f : hs[(int64_t)(K - 1 + row - c0) * W + c];
+          v = (X[(int64_t)row * W + c] - s_mean[si]) * s_rstd[si] * wc;
+        } else if (!fresh) {
+          v = hs[(int64_t)(K - 1 + row - c0) * W + c];
         }
-        acc += tc[j] * hv;
-        self = hv;
       }
-      stf<T>(out, (int64_t)(tok0 + i) * W + c, self + acc);
+      hv[m] = v;
+    }
+    for (int i = 0; i < n; ++i) {
+      const int row = tok0 + i, si = row - r_lo;
+      const float self =
+          (X[(int64_t)row * W + c] - s_mean[si]) * s_rstd[si] * wc;
+      float acc = tw[MAXK - 1] * self;
+#pragma unroll
+      for (int m = 0; m < MAXK - 1; ++m) acc += tw[m] * hv[m];
+#pragma unroll
+      for (int m = 0; m < MAXK - 2; ++m) hv[m] = hv[m + 1];
+      hv[MAXK - 2] = self;
+      stf<T>(out, (int64_t)row * W + c, self + acc);
     }
   }
   if (!first || K <= 1) return;
@@ -192,6 +211,42 @@ __global__ __launch_bounds__(BLOCK) void postln_add_kernel(
   float* xr = X + row * W;
   for (int c = threadIdx.x; c < W; c += BLOCK)
     xr[c] += (u[c] - mu) * rs * w[c];
+}
+
+// bf16 rows whose length is a multiple of 8: 16-byte loads and stores
+__global__ __launch_bounds__(BLOCK) void polynorm_vec8_kernel(
+    const bf16* __restrict__ z, const float* __restrict__ coef,
+    bf16* __restrict__ out, int N, float eps) {
+  __shared__ float r1[NW], r2[NW], r3[NW];
+  const int64_t row = blockIdx.x;
+  const bf16x8* zr = reinterpret_cast<const bf16x8*>(z + row * N);
+  bf16x8* orow = reinterpret_cast<bf16x8*>(out + row * N);
+  float a = 0.f, b = 0.f, c3 = 0.f;
+  for (int c = threadIdx.x; c < N / 8; c += BLOCK) {
+    const bf16x8 v8 = zr[c];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = bf2f(v8.v[e]), v2 = v * v;
+      a += v2;
+      b += v2 * v2;
+      c3 += v2 * v2 * v2;
+    }
+  }
+  const float n1 = 1.0f / sqrtf(block_reduce_sum<NW>(a, r1) / (float)N + eps);
+  const float n2 = 1.0f / sqrtf(block_reduce_sum<NW>(b, r2) / (float)N + eps);
+  const float n3 = 1.0f / sqrtf(block_reduce_sum<NW>(c3, r3) / (float)N + eps);
+  const float k1 = coef[0] * n1, k2 = coef[1] * n2, k3 = coef[2] * n3,
+              k0 = coef[3];
+  for (int c = threadIdx.x; c < N / 8; c += BLOCK) {
+    const bf16x8 v8 = zr[c];
+    bf16x8 o8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = bf2f(v8.v[e]), v2 = v * v;
+      o8.v[e] = f2bf(k1 * v + k2 * v2 + k3 * v2 * v + k0);
+    }
+    orow[c] = o8;
+  }
 }
 
 template <typename T>
@@ -304,6 +359,10 @@ void tl_polynorm(const void* z, const void* coef, void* out, int64_t rows,
     hipLaunchKernelGGL(polynorm_kernel<float>, dim3(rows), dim3(BLOCK), 0,
                        stream, (const float*)z, (const float*)coef,
                        (float*)out, N, eps);
+  else if (N % 8 == 0)
+    hipLaunchKernelGGL(polynorm_vec8_kernel, dim3(rows), dim3(BLOCK), 0,
+                       stream, (const bf16*)z, (const float*)coef, (bf16*)out,
+                       N, eps);
   else
     hipLaunchKernelGGL(polynorm_kernel<bf16>, dim3(rows), dim3(BLOCK), 0,
                        stream, (const bf16*)z, (const float*)coef, (bf16*)out,

@@ -822,6 +822,33 @@ def ssd_scan(xbc: torch.Tensor, offs, dt_src: torch.Tensor, dt_col: int,
     assert xbc.dtype == torch.float32 and S.dtype == torch.float32
     assert S.shape[1:] == (H, N, P) and H % G == 0
     if xbc.is_cuda:
+        chunk = SCAN_CHUNK
+        while meta.T * H * N * P * 4 // chunk > (1 << 31):
+            chunk *= 2                   # bound the chunk-state scratch
+        if (max(meta.new_h) >= 4 * chunk
+                and not os.environ.get("TL_NO_SCAN_CHUNKS")):
+            # long prompt portions: chunk form. The intra-chunk part
+            # (C B^T with the decay mask, times dt x), the chunk summary
+            # Bw^T (dt x) and the carried part Cd S0 are batched fp32 GEMMs
+            # over all chunks at once; only the chain of summaries is
+            # sequential.
+            C = _ext()
+            cu_c, _, _, base, cnt, nc, _ = meta.scan_chunks(chunk)
+            Cs, Cd, Bs, Bw, Xd, Lc, tot = C.ssd_chunk_prep(
+                xbc, int(x_off), int(b_off), int(c_off), dt_src, int(dt_col),
+                dt_bias, A_log, cu_c, int(H), int(P), int(N), int(G), chunk)
+            A = torch.bmm(Cs, Bs.transpose(1, 2))
+            C.ssd_decay_mask_(A, Lc)
+            O = torch.bmm(A, Xd)
+            U = torch.bmm(Bw.transpose(1, 2), Xd)
+            C.ssd_chain_(U, S, tot, base, cnt, meta.slots, meta.pos0)
+            O.baddbmm_(Cd, U)
+            y = O.view(nc, H, chunk, P).transpose(1, 2).reshape(
+                nc * chunk, H * P).index_select(0, meta.chunk_rows(chunk))
+            y.view(T, H, P).addcmul_(
+                xbc[:, x_off:x_off + H * P].view(T, H, P),
+                skip.view(1, H, 1))
+            return y
         return _ext().ssd_scan(xbc, int(x_off), int(b_off), int(c_off),
                                dt_src, int(dt_col), dt_bias, A_log, skip, S,
                                meta.cu, meta.slots, meta.pos0, int(H),
