@@ -752,11 +752,11 @@ def random_cfg(rng):
     return cfg
 
 
-@pytest.mark.parametrize("device,dtype", [CPU32, GPU32])
+@pytest.mark.parametrize("device,dtype", ALL)
 def test_random_configurations(tmp_path, device, dtype):
     """Other sizes, orders and constants: whole, portioned and decoded
     against the oracle."""
-    for seed in (1, 2, 3, 4, 5, 6):
+    for seed in (1, 2, 3, 4, 5, 6, 7, 8):
         cfg = random_cfg(random.Random(seed))
         P = make_weights(cfg, seed)
         d = str(tmp_path / f"r{seed}")
@@ -769,8 +769,11 @@ def test_random_configurations(tmp_path, device, dtype):
         for cuts in ([140], [90, 2, 3, 40]):
             got = run_schedule(batcher(runner, max_ctx=256), toks, cuts)
             e = rel_err(got, want)
-            assert float(e.median()) < 2e-5 and float(e.max()) < 1e-3, \
-                (seed, cuts, float(e.median()), float(e.max()))
+            if dtype == torch.float32:
+                assert float(e.median()) < 2e-5 and float(e.max()) < 1e-3, \
+                    (seed, cuts, float(e.median()), float(e.max()))
+            else:
+                assert close(got, want, dtype), (seed, cuts)
 
 
 # --------------------------------------------------- configuration, loader
