@@ -14,7 +14,8 @@
 // `pool` (rotated) and, when given, of `raw_pool` (as they leave the
 // convolution: a value pool that shares the key projection).
 //
-// One block per tile of <= TILE tokens of one sequence. A work item is a
+// One block per tile of <= TILE tokens of one sequence (with few tiles the
+// work items of a tile are spread over several blocks). A work item is a
 // rotated pair or a single unrotated channel, so rotation needs no
 // exchange between threads; the tile's cos/sin table is built once in LDS
 // and shared by all heads. TILE >= K-1, so only the block of a portion's
@@ -70,7 +71,10 @@ __global__ __launch_bounds__(BLOCK) void conv_rope_rows_kernel(
   float* hs = hist + (int64_t)slots[seq] * (K - 1) * N;
   const int iph = D - half;         // work items per head
   const int* tab = table + (int64_t)seq * P;
-  for (int e = threadIdx.x; e < n_heads * iph; e += BLOCK) {
+  // few tiles (decoding): the work items are spread over gridDim.y blocks
+  const int e_first = blockIdx.y * BLOCK + threadIdx.x;
+  const int e_step = gridDim.y * BLOCK;
+  for (int e = e_first; e < n_heads * iph; e += e_step) {
     const int hd = e / iph, r = e - hd * iph;
     const bool pair = r < half;
     const int d0 = pair ? r : r + half;
@@ -152,15 +156,22 @@ __global__ __launch_bounds__(BLOCK) void conv_rope_rows_kernel(
   }
   if (!first || K <= 1) return;
   __syncthreads();       // every read of the old history is done
-  for (int c = threadIdx.x; c < N; c += BLOCK) {
-    for (int r = 0; r < K - 1; ++r) {
-      const int rr = ntot - (K - 1) + r;
-      float v;
-      if (rr >= 0)
-        v = ldf<T>(src, (int64_t)(c0 + rr) * ld + col + c);
-      else      // ascending r: source index r + ntot is not yet overwritten
-        v = fresh ? 0.f : hs[(int64_t)(r + ntot) * N + c];
-      hs[(int64_t)r * N + c] = v;
+  // a block updates the channels of its own work items
+  for (int e = e_first; e < n_heads * iph; e += e_step) {
+    const int hd = e / iph, r = e - hd * iph;
+    const bool pair = r < half;
+    const int ch0 = hd * D + (pair ? r : r + half);
+    for (int k = 0; k < (pair ? 2 : 1); ++k) {
+      const int c = ch0 + k * half;
+      for (int r2 = 0; r2 < K - 1; ++r2) {
+        const int rr = ntot - (K - 1) + r2;
+        float v;
+        if (rr >= 0)
+          v = ldf<T>(src, (int64_t)(c0 + rr) * ld + col + c);
+        else    // ascending: source index r2 + ntot is not yet overwritten
+          v = fresh ? 0.f : hs[(int64_t)(r2 + ntot) * N + c];
+        hs[(int64_t)r2 * N + c] = v;
+      }
     }
   }
 }
@@ -185,8 +196,11 @@ int tl_conv_rope_rows(const void* src, int ld, int col, int n_heads, int D,
     return 1;
   const size_t smem = sizeof(float) * 2 * TILE * (size_t)(rot_dims / 2);
   if (smem > 64 * 1024) return 1;
+  const int items = n_heads * (D - rot_dims / 2);
+  const int gy = n_tiles >= 512 ? 1 : min(16, max(1, (items + BLOCK - 1) / BLOCK));
+  const dim3 grid(n_tiles, gy);
   if (is_f32)
-    hipLaunchKernelGGL(conv_rope_rows_kernel<float>, dim3(n_tiles),
+    hipLaunchKernelGGL(conv_rope_rows_kernel<float>, grid,
                        dim3(BLOCK), smem, stream, (const float*)src, ld, col,
                        n_heads, D, (const float*)taps, (const float*)bias,
                        act_silu, (float*)hist, K, rot_dims,
@@ -195,7 +209,7 @@ int tl_conv_rope_rows(const void* src, int ld, int col, int n_heads, int D,
                        (const int*)table, P, (float*)out, (float*)pool,
                        (float*)raw_pool, pool_heads);
   else
-    hipLaunchKernelGGL(conv_rope_rows_kernel<bf16>, dim3(n_tiles),
+    hipLaunchKernelGGL(conv_rope_rows_kernel<bf16>, grid,
                        dim3(BLOCK), smem, stream, (const bf16*)src, ld, col,
                        n_heads, D, (const float*)taps, (const float*)bias,
                        act_silu, (float*)hist, K, rot_dims,

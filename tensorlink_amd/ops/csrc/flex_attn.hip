@@ -26,6 +26,8 @@
 
 #include "common.hpp"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int PAGE = 128;
@@ -133,13 +135,18 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
   }
   __syncthreads();
 
-  float m[HB], l[HB], a[HB][VR];
+  // VR == 0: value rows are fetched with 16-byte loads (bf16 pools, value
+  // size 8 * 2^k): CPR lanes cover one row, so one load instruction brings
+  // 64 / CPR rows; a lane accumulates 8 columns for the keys of its row
+  // group and the row groups meet through shuffles at the end
+  constexpr int AC = VR == 0 ? 8 : VR;
+  float m[HB], l[HB], a[HB][AC];
 #pragma unroll
   for (int b = 0; b < HB; ++b) {
     m[b] = -INFINITY;
     l[b] = 0.f;
 #pragma unroll
-    for (int r = 0; r < VR; ++r) a[b][r] = 0.f;
+    for (int r = 0; r < AC; ++r) a[b][r] = 0.f;
   }
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int first = (lo / WAVE_SIZE) * WAVE_SIZE;
@@ -191,19 +198,48 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       l[b] = l[b] * c + wave_reduce_sum(p[b]);
       m[b] = nm;
 #pragma unroll
-      for (int r = 0; r < VR; ++r) a[b][r] *= c;
+      for (int r = 0; r < AC; ++r) a[b][r] *= c;
     }
     const int jb = max(0, lo - j0), je = min(WAVE_SIZE, pos + 1 - j0);
     const TK* vtile = vpool + (page_row + (int64_t)g0 * PAGE) * vld;
+    if constexpr (VR == 0) {
+      const int CPR = V >> 3, KGR = WAVE_SIZE / CPR;
+      const int cc = lane & (CPR - 1), kg = lane / CPR;
+      for (int jj0 = jb; jj0 < je; jj0 += 4 * KGR) {
+        bf16x8 vv[4];
+        int jk[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          jk[u] = jj0 + u * KGR + kg;
+          if (jk[u] < je)
+            vv[u] = *reinterpret_cast<const bf16x8*>(
+                vtile + (int64_t)jk[u] * vld + cc * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const bool on = jk[u] < je;
+          const int src = min(jk[u], WAVE_SIZE - 1);
+#pragma unroll
+          for (int b = 0; b < HB; ++b) {
+            const float ws = __shfl(p[b], src, WAVE_SIZE);
+            if (on) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) a[b][e] += ws * bf2f(vv[u].v[e]);
+            }
+          }
+        }
+      }
+      continue;
+    }
     // eight keys' value rows are loaded before they are used, so their
     // latencies overlap instead of adding up
     for (int jj0 = jb; jj0 < je; jj0 += 8) {
-      float vv[8][VR];
+      float vv[8][AC];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const TK* vr = vtile + (int64_t)(jj0 + u) * vld;
 #pragma unroll
-        for (int r = 0; r < VR; ++r) {
+        for (int r = 0; r < AC; ++r) {
           const int c = lane + r * WAVE_SIZE;
           vv[u][r] = (jj0 + u < je && c < V) ? ldv<TK>(vr + c) : 0.f;
         }
@@ -216,7 +252,7 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
         for (int b = 0; b < HB; ++b) {
           const float w = jj0 + u < je ? __shfl(p[b], jj, WAVE_SIZE) : 0.f;
 #pragma unroll
-          for (int r = 0; r < VR; ++r) a[b][r] += w * vv[u][r];
+          for (int r = 0; r < AC; ++r) a[b][r] += w * vv[u][r];
         }
       }
     }
@@ -228,10 +264,21 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       stat[(wave * HB + b) * 2 + 0] = m[b];
       stat[(wave * HB + b) * 2 + 1] = l[b];
     }
+    if constexpr (VR == 0) {
+      const int CPR = V >> 3;
 #pragma unroll
-    for (int r = 0; r < VR; ++r) {
-      const int c = lane + r * WAVE_SIZE;
-      if (c < V) accs[(wave * HB + b) * V + c] = a[b][r];
+      for (int e = 0; e < 8; ++e) {
+        float s = a[b][e];
+        for (int off = CPR; off < WAVE_SIZE; off <<= 1)
+          s += __shfl_xor(s, off, WAVE_SIZE);
+        if (lane < CPR) accs[(wave * HB + b) * V + lane * 8 + e] = s;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < AC; ++r) {
+        const int c = lane + r * WAVE_SIZE;
+        if (c < V) accs[(wave * HB + b) * V + c] = a[b][r];
+      }
     }
   }
   __syncthreads();
@@ -390,6 +437,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       const void* sinks, hipStream_t stream) {
   if (T <= 0) return 0;
   const bool has_talk = talk != nullptr;
+  static const bool no_vec = getenv("TL_NO_VEC_VALUES") != nullptr;
   const int hb = heads_per_block(H, G, DK, V, has_talk ? 1 : 0, hb_max);
   if (hb == 0 || ns < 1 || (ns > 1 && !part)) return 1;
   const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
@@ -412,8 +460,17 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
   else if (hb == 4) { TL_FA_V(TT, 4) } \
   else if (hb == 2) { TL_FA_V(TT, 2) } \
   else { TL_FA_V(TT, 1) }
+  // 16-byte value loads: bf16 rows of 8 * 2^k columns, 16-byte aligned
+  const int cpr = V / 8;
+  const bool vec = !pool_f32 && V % 8 == 0 && cpr >= 1 && cpr <= WAVE_SIZE &&
+                   (cpr & (cpr - 1)) == 0 && vld % 8 == 0 && !no_vec;
   if (pool_f32) {
     TL_FA_H(float)
+  } else if (vec) {
+    if (hb == 8) TL_FA(bf16, 8, 0);
+    else if (hb == 4) TL_FA(bf16, 4, 0);
+    else if (hb == 2) TL_FA(bf16, 2, 0);
+    else TL_FA(bf16, 1, 0);
   } else {
     TL_FA_H(bf16)
   }

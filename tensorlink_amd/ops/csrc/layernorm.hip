@@ -116,7 +116,11 @@ __global__ __launch_bounds__(BLOCK) void ln_canon_kernel(
   }
   __syncthreads();
   float* hs = hist + (int64_t)slots[seq] * (K - 1) * W;
-  for (int c = threadIdx.x; c < W; c += BLOCK) {
+  // few tiles (decoding): the channels are spread over gridDim.y blocks,
+  // each with its own copy of the row statistics
+  const int c_first = blockIdx.y * BLOCK + threadIdx.x;
+  const int c_step = gridDim.y * BLOCK;
+  for (int c = c_first; c < W; c += c_step) {
     const float wc = w[c];
     // taps and the sliding window of normed values are aligned at the END
     // of fixed-size arrays (leading entries zero): every index is static
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(BLOCK) void ln_canon_kernel(
   }
   if (!first || K <= 1) return;
   __syncthreads();       // every read of the old history is done
-  for (int c = threadIdx.x; c < W; c += BLOCK) {
+  for (int c = c_first; c < W; c += c_step) {
     const float wc = w[c];
     for (int r = 0; r < K - 1; ++r) {
       const int rr = ntot - (K - 1) + r;        // row within the portion
@@ -321,14 +325,16 @@ void tl_ln_canon(const void* X, const void* w, const void* taps, void* hist,
                  const void* slots, const void* pos0, void* out, int W, int K,
                  float eps, int out_f32, hipStream_t stream) {
   if (n_tiles <= 0) return;
+  const int gy = n_tiles >= 512 ? 1 : min(8, max(1, (W + BLOCK - 1) / BLOCK));
+  const dim3 grid(n_tiles, gy);
   if (out_f32)
-    hipLaunchKernelGGL(ln_canon_kernel<float>, dim3(n_tiles), dim3(BLOCK), 0,
+    hipLaunchKernelGGL(ln_canon_kernel<float>, grid, dim3(BLOCK), 0,
                        stream, (const float*)X, (const float*)w,
                        (const float*)taps, (float*)hist, (const int*)tiles,
                        (const int*)cu, (const int*)slots, (const int*)pos0,
                        (float*)out, W, K, eps);
   else
-    hipLaunchKernelGGL(ln_canon_kernel<bf16>, dim3(n_tiles), dim3(BLOCK), 0,
+    hipLaunchKernelGGL(ln_canon_kernel<bf16>, grid, dim3(BLOCK), 0,
                        stream, (const float*)X, (const float*)w,
                        (const float*)taps, (float*)hist, (const int*)tiles,
                        (const int*)cu, (const int*)slots, (const int*)pos0,
