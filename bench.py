@@ -229,10 +229,10 @@ def dizepel_configs(z):
     mixer = {
         "left": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"],
                  "vdim": z["dim"], "conv": 4, "scale": z["dim"] ** -0.5,
-                 "softcap": 50.0,
-                 "rot": {"dims": z["rot"], "base": 250000.0,
-                         "scaling": {"factor": 4.0, "original": 2048,
-                                     "fast": 32.0, "slow": 1.0}}},
+                 "softcap": 30.0,
+                 "rot": {"dims": z["rot"], "base": 500000.0,
+                         "scaling": {"factor": 8.0, "original": 2048,
+                                     "fast": 16.0, "slow": 2.0}}},
         "right": {"heads": z["ssm_heads"], "vdim": z["ssm_dim"],
                   "state": z["state"], "groups": z["groups"], "conv": 4,
                   "norm_groups": z["groups"]}}
@@ -241,7 +241,7 @@ def dizepel_configs(z):
     diz = DizepelConfig.from_dict({
         "architecture": "Dizepel", "vocab": z["vocab"], "width": z["width"],
         "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
-        "canon": {"taps": 3}, "loop": {"start": 2, "stop": 4, "times": 2},
+        "canon": {"taps": 4}, "loop": {"start": 2, "stop": 4, "times": 2},
         "layers": [layer] * 6}, name="dizepel-" + str(z["width"]))
     ref = ModelConfig(
         name="dense-gqa-" + str(z["width"]), vocab_size=z["vocab"],

@@ -114,8 +114,8 @@ def cfg_tiles():
     multiple of 8 and of 16): the capped scores and the sinks of that
     kernel; the loop at the model's end."""
     return {"architecture": "Dizepel", "vocab": 70, "width": 64,
-            "norm": {"eps": 1e-5}, "embedding": {"scale": 3.0},
-            "canon": {"taps": 3},
+            "norm": {"eps": 1e-5}, "embedding": {"scale": 0.5},
+            "canon": {"taps": 5},
             "loop": {"start": 1, "stop": 2, "times": 2},
             "layers": [
                 par(left(4, 2, 32, conv=4, rot=16, scaling=YARN,
