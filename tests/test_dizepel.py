@@ -7,7 +7,6 @@ framework's stage, cache and batcher. The same bodies run on the CPU tier
 """
 
 import json
-import math
 import os
 import random
 
@@ -16,7 +15,6 @@ import torch
 
 import dizepel_oracle as O
 from tensorlink_amd.engine.batcher import ContinuousBatcher
-from tensorlink_amd.models import mixers as M
 from tensorlink_amd.models.paged import PAGE, HybridSlotCache
 from tensorlink_amd.ops import mixers as mx
 from tensorlink_amd.parallel.pipeline import PipelineRunner, SamplingParams
