@@ -1,5 +1,5 @@
 """Dizepel model family: a layered decoder whose ``config.json`` lists
-every layer. A layer's mixer is two mixers side by side on the same input
+every layer. A layer's mixer is a pair of mixers fed by the same input
 — softmax attention with short convolutions, a learned sink and capped
 scores whose values are its unrotated keys, and a selective state-space
 (SSD) mixer — followed by an optional PolyNorm feed-forward. Every

@@ -470,7 +470,8 @@ class TokenSide(nn.Module):
 # blocks of the parallel-mixer family: layer norm without bias, causal
 # input convolution, softmax attention with short convolutions / a learned
 # sink / capped scores whose values are its unrotated keys, a selective
-# state-space (SSD) mixer, the two side by side, and a PolyNorm feed-forward
+# state-space (SSD) mixer, a pair of mixers on one input, and a PolyNorm
+# feed-forward
 # ---------------------------------------------------------------------------
 class LayerNormWeight(nn.Module, _F32Cache):
     """Weight of a layer norm without bias."""
@@ -506,7 +507,7 @@ class ConvSinkAttention(nn.Module, _F32Cache):
     ``rot_dims`` dimensions of every head (optionally with a two-regime
     frequency scaling, see ``ops.mixers.yarn_freqs``); scores are scaled,
     optionally capped through tanh, and the softmax denominator holds one
-    learned logit per head (``sink``) that has no key and no value.
+    learned logit per head (``sink``): weight that attends to nothing.
 
     The module owns everything after the input projection; ``in_cols``
     columns [q | k] of the caller's projection feed it. Per-sequence
@@ -606,7 +607,7 @@ class SSDMixer(nn.Module, _F32Cache):
 
 
 class ParallelMixer(nn.Module, _F32Cache):
-    """Two mixers side by side on the same input: ``left`` (attention) and
+    """A pair of mixers fed by the same input: ``left`` (attention) and
     ``right`` (state-space), fed by ONE fused input projection. The result
     is half the sum of the two outputs after each is RMS-normed over the
     model width with its plain weight (``left_out`` / ``right_out``);

@@ -11,8 +11,8 @@
 // formed in double, cos and sin times `mult`. The first n_heads -
 // pool_heads heads are written densely in fp32 (queries, or the inputs of a
 // recurrence); the last pool_heads heads go to the tokens' page rows of
-// `pool` (rotated) and, when given, of `raw_pool` (as they leave the
-// convolution: a value pool that shares the key projection).
+// `pool` (rotated) and, when given, of `raw_pool` (the unrotated
+// convolution output: a value pool that shares the key projection).
 //
 // One block per tile of <= TILE tokens of one sequence (with few tiles the
 // work items of a tile are spread over several blocks). A work item is a

@@ -6,8 +6,8 @@
 //     dt_t = softplus(r_t + dt_bias_h)
 //     S_t  = exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T   (S: [N, P])
 //     y_t  = S_t^T C_t + skip_h x_t
-// x [H*P], B [G*N], C [G*N] arrive in fp32 (they leave the convolution
-// kernel so); softplus, exponentials, the state and the read-out are fp32.
+// x [H*P], B [G*N], C [G*N] arrive in fp32 (the convolution kernel writes
+// them so); softplus, exponentials, the state and the read-out are fp32.
 // One block per (sequence, head) walks the sequence's new tokens in order;
 // the state comes from the sequence's slot (zeros when it has no cached
 // tokens) and goes back there, so prompt portions of any size and single

@@ -733,7 +733,7 @@ def conv_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
     [T, (n_heads - pool_heads)*head_dim]; the last ``pool_heads`` heads
     are scattered to the tokens' page rows of ``pool``
     [pages, pool_heads, PAGE, head_dim] after rotation and, with
-    ``raw_pool``, as they leave the convolution (before rotation) too."""
+    ``raw_pool``, the unrotated convolution output as well."""
     N = n_heads * head_dim
     T = src.shape[0]
     K = conv_w.shape[1]
