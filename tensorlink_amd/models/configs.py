@@ -119,6 +119,9 @@ class ModelConfig:
         if cfg.get("architecture") in ("Dizepel", "dizepel"):
             from tensorlink_amd.models.dizepel import DizepelConfig
             return DizepelConfig.from_dict(cfg, name=name)
+        if cfg.get("architecture") in ("Potosun", "potosun"):
+            from tensorlink_amd.models.potosun import PotosunConfig
+            return PotosunConfig.from_dict(cfg, name=name)
         if "architecture" in cfg and "architectures" not in cfg:
             # our own to_json round-trip (save_hf_checkpoint writes it)
             known = {f.name for f in dataclasses.fields(cls)}

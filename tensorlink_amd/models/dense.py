@@ -460,4 +460,7 @@ def _stage_class(config: ModelConfig):
     if config.architecture == "dizepel":
         from tensorlink_amd.models.dizepel import DizepelStageModel
         return DizepelStageModel
+    if config.architecture == "potosun":
+        from tensorlink_amd.models.potosun import PotosunStageModel
+        return PotosunStageModel
     return StageModel

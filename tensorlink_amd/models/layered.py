@@ -70,6 +70,22 @@ class LayeredStage(nn.Module):
         return self.embed_tokens(input_ids)
 
 
+def tensor_shapes(ckpt_dir: str) -> Dict[str, Tuple[int, ...]]:
+    """Tensor name -> shape from the header of ``model.safetensors`` in
+    ``ckpt_dir`` (an 8-byte little-endian length, then that many bytes of
+    JSON); no tensor data is read. Empty if there is no such file."""
+    import json
+    import struct
+    path = os.path.join(ckpt_dir, "model.safetensors")
+    if not os.path.isfile(path):
+        return {}
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in header.items()
+            if k != "__metadata__"}
+
+
 @torch.no_grad()
 def load_named_tensors(params: Dict[str, torch.Tensor],
                        names: Dict[str, Tuple[str, int]], ckpt_dir: str,

@@ -137,6 +137,11 @@ def load_stage_from_checkpoint(stage: StageModel, ckpt_dir: str,
         n = load_dizepel_weights(stage, ckpt_dir, dtype=dtype)
         stage.to(device=device, dtype=dtype)
         return n
+    if arch == "potosun":
+        from tensorlink_amd.models.potosun import load_potosun_weights
+        n = load_potosun_weights(stage, ckpt_dir, dtype=dtype)
+        stage.to(device=device, dtype=dtype)
+        return n
     from safetensors import safe_open
 
     index_path = os.path.join(ckpt_dir, "model.safetensors.index.json")
@@ -187,6 +192,10 @@ def init_random_stage(stage: StageModel, device="cpu", dtype=torch.bfloat16,
     if stage.config.architecture == "dizepel":
         from tensorlink_amd.models.dizepel import init_dizepel_random
         init_dizepel_random(stage, seed=seed)
+        return stage.to(device=device, dtype=dtype)
+    if stage.config.architecture == "potosun":
+        from tensorlink_amd.models.potosun import init_potosun_random
+        init_potosun_random(stage, seed=seed)
         return stage.to(device=device, dtype=dtype)
     gen_dev = device if str(device).startswith("cuda") else "cpu"
     g = torch.Generator(device=gen_dev)

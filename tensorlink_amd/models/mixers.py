@@ -311,22 +311,37 @@ class LatentAttention(nn.Module, _F32Cache):
     of the row); W_uv is applied to the attended latent afterwards. The
     per-head keys and values are never materialised. ``kv_from`` = index
     of an earlier latent layer whose cached rows this layer reads with its
-    own W_uk / W_uv and queries."""
+    own W_uk / W_uv and queries.
+
+    Options: ``window`` > 0 = sliding window; ``rot_scaling`` = two-regime
+    frequency scaling of the rotation (see ``ops.mixers.yarn_freqs``);
+    ``sink_logits`` = one learned logit per head in the softmax denominator
+    (``sink``); ``head_gate`` = head h's output times sigmoid of one more
+    projection of the input (``g`` rows of the fused projection, one per
+    head). A scalar gate commutes with W_uv, so it is applied to the
+    attended latent where the attention kernel writes it."""
 
     kind = "latent_attention"
 
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int,
                  vdim: int, kv_rank: int, scale: float, rot_base: float,
-                 eps: float, kv_from: Optional[int] = None):
+                 eps: float, kv_from: Optional[int] = None, *,
+                 window: int = 0, rot_scaling: Optional[dict] = None,
+                 sink_logits: bool = False, head_gate: bool = False):
         super().__init__()
         assert rot_dim % 2 == 0
         self.H, self.D, self.RD, self.V, self.R = (heads, dim, rot_dim, vdim,
                                                    kv_rank)
         self.scale, self.eps, self.base = float(scale), float(eps), rot_base
         self.kv_from = kv_from
+        self.window = int(window)
+        self.rot_scaling = dict(rot_scaling) if rot_scaling else None
         self.q_cols = heads * (dim + rot_dim)
         self.kv_cols = 0 if kv_from is not None else kv_rank + rot_dim
-        self.qdkv = TLLinear(width, self.q_cols + self.kv_cols, bias=False)
+        self.g_cols = heads if head_gate else 0
+        self.qdkv = TLLinear(width, self.q_cols + self.kv_cols + self.g_cols,
+                             bias=False)
+        self.sink = nn.Parameter(torch.zeros(heads)) if sink_logits else None
         if kv_from is None:
             self.dkv_norm = nn.Parameter(torch.ones(kv_rank))
         self.uk = nn.Parameter(torch.zeros(heads * dim, kv_rank))
@@ -339,33 +354,39 @@ class LatentAttention(nn.Module, _F32Cache):
         return {"kind": "kv", "G": 1, "DK": self.R + self.RD, "V": 0}
 
     def _freqs(self, dev):
+        """(frequencies, multiplier of cos and sin)."""
         hit = self.__dict__.get("_fr")
-        if hit is None or hit.device != dev:
-            hit = mx.rope_freqs(self.RD, self.base, dev)
+        if hit is None or hit[0].device != dev:
+            hit = mx.yarn_freqs(self.RD, self.base, self.rot_scaling, dev)
             self.__dict__["_fr"] = hit
         return hit
 
-    def forward(self, h, meta, cache, layer_idx):
+    def forward(self, h, meta, cache, layer_idx, shared=None):
         H, D, RD, R, V = self.H, self.D, self.RD, self.R, self.V
         T = h.shape[0]
         proj = self.qdkv(h)
-        fr = self._freqs(h.device)
+        fr, mult = self._freqs(h.device)
         src = layer_idx if self.kv_from is None else self.kv_from
         pool = cache.k[src]
         if self.kv_from is None:
             mx.norm_rope_rows(proj, self.q_cols, 1, R + RD, meta,
                               norm_w=self._f32("dkv_norm"), norm_cols=R,
                               eps=self.eps, rot_off=R, rot_dims=RD,
-                              freqs=fr, pool=pool)
+                              freqs=fr, rot_mult=mult, pool=pool)
         q = mx.norm_rope_rows(proj, 0, H, D + RD, meta, rot_off=D,
-                              rot_dims=RD, freqs=fr).view(T, H, D + RD)
+                              rot_dims=RD, freqs=fr,
+                              rot_mult=mult).view(T, H, D + RD)
         qa = torch.empty(T, H, R + RD, device=h.device, dtype=torch.float32)
         qa[:, :, R:] = q[:, :, D:]
         torch.bmm(q[:, :, :D].transpose(0, 1),
                   self._f32("uk").view(H, D, R),
                   out=qa[:, :, :R].transpose(0, 1))
-        o = mx.flex_attention(qa.view(T, H * (R + RD)), pool, None, meta, H,
-                              self.scale, v_cols=R)
+        o = mx.flex_attention(
+            qa.view(T, H * (R + RD)), pool, None, meta, H, self.scale,
+            v_cols=R, window=self.window,
+            sink_logits=self._f32("sink") if self.sink is not None else None,
+            gate=proj if self.g_cols else None,
+            gate_col=self.q_cols + self.kv_cols, gate_heads=True)
         o = torch.bmm(o.view(T, H, R).transpose(0, 1),
                       self._f32("uv").view(H, V, R).transpose(1, 2))
         return self.o_proj(o.transpose(0, 1).reshape(T, H * V).to(h.dtype))
@@ -378,28 +399,70 @@ class WindowAttention(nn.Module, _F32Cache):
     the first ``rot_dims`` dimensions of every head; a learned [H, H]
     mixing of the heads' scores before the softmax (``talk``); a sliding
     window (``window`` = 0: plain causal); a sink (one added to the
-    softmax denominator)."""
+    softmax denominator).
+
+    Further options, all off by default:
+    ``head_norm``    the query / key norm is per head over ``dim`` with one
+                     weight [dim] shared by the heads;
+    ``interleaved``  rotation pairs are (2i, 2i+1) instead of halves;
+    ``chunk``        instead of a window: a query sees the keys of its own
+                     chunk of this many positions, counted from position 0;
+    ``keep_first``   the first positions stay visible beyond the window;
+    ``sink_logits``  a learned logit per head in the denominator (``sinks``)
+                     instead of the constant one;
+    ``rel_rows``, ``rel_far``  a learned distance bias ``rel``
+                     [rel_rows, heads] added to the scaled score, distances
+                     bucketed exactly up to rel_rows / 2 and geometrically up
+                     to ``rel_far`` (``ops.mixers.log_distance_buckets``);
+    ``out_gate``     the concatenated heads times sigmoid of one more
+                     projection of the input (``g`` rows of the fused
+                     projection);
+    ``v_mix``        value mixing across layers: the first such layer of a
+                     model publishes its values of the step's tokens in the
+                     ``shared`` dictionary handed to forward, later ones
+                     cache (1 - vmix) v + vmix v_first (``vmix`` a learned
+                     scalar); the mixing layers must agree in kv_heads *
+                     vdim."""
 
     kind = "attention"
 
     def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
                  vdim: int, scale: float, rot_dims: int, rot_base: float,
                  window: int, eps: float, sink: bool = True,
-                 talk: bool = True, qk_norm: bool = True):
+                 talk: bool = True, qk_norm: bool = True, *,
+                 head_norm: bool = False, interleaved: bool = False,
+                 chunk: int = 0, keep_first: int = 0,
+                 sink_logits: bool = False, rel_rows: int = 0,
+                 rel_far: float = 0.0, out_gate: bool = False,
+                 v_mix: bool = False):
         super().__init__()
         assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim
+        assert not (chunk and window), "a chunked mask has no window"
         self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
         self.scale, self.eps = float(scale), float(eps)
         self.rot_dims, self.base = int(rot_dims), rot_base
-        self.window, self.sink = int(window), bool(sink)
+        self.window, self.sink = int(window), bool(sink or sink_logits)
+        self.head_norm, self.interleaved = bool(head_norm), bool(interleaved)
+        self.chunk, self.keep_first = int(chunk), int(keep_first)
+        self.rel_rows, self.rel_far = int(rel_rows), float(rel_far)
+        self.v_mix = bool(v_mix)
         self.q_cols, self.k_cols = heads * dim, kv_heads * dim
-        self.qkv = TLLinear(width, self.q_cols + self.k_cols
-                            + kv_heads * vdim, bias=False)
-        self.q_norm = nn.Parameter(torch.ones(self.q_cols)) if qk_norm \
-            else None
-        self.k_norm = nn.Parameter(torch.ones(self.k_cols)) if qk_norm \
-            else None
+        self.v_cols = kv_heads * vdim
+        self.g_cols = heads * vdim if out_gate else 0
+        self.qkv = TLLinear(width, self.q_cols + self.k_cols + self.v_cols
+                            + self.g_cols, bias=False)
+        self.q_norm = nn.Parameter(torch.ones(
+            dim if head_norm else self.q_cols)) if qk_norm else None
+        self.k_norm = nn.Parameter(torch.ones(
+            dim if head_norm else self.k_cols)) if qk_norm else None
         self.talk = nn.Parameter(torch.eye(heads)) if talk else None
+        self.sinks = nn.Parameter(torch.zeros(heads)) if sink_logits \
+            else None
+        self.rel = nn.Parameter(torch.zeros(rel_rows, heads)) if rel_rows \
+            else None
+        self.vmix = nn.Parameter(torch.zeros(())) if v_mix else None
+        if rel_rows:
+            self.buckets = mx.log_distance_buckets(rel_rows, rel_far)
         self.o_proj = TLLinear(heads * vdim, width, bias=False)
 
     def cache_spec(self):
@@ -412,25 +475,62 @@ class WindowAttention(nn.Module, _F32Cache):
             self.__dict__["_fr"] = hit
         return hit
 
-    def forward(self, h, meta, cache, layer_idx):
+    def _dist_bias(self, dev):
+        """The distance bias spread over distances: fp32 [H, n] with
+        entry [h, d] = rel[bucket(d), h]; the last column serves every
+        larger distance. Rebuilt when ``rel`` changes."""
+        p = self.rel
+        key = (p.data_ptr(), p._version, p.device)
+        hit = self.__dict__.get("_lut")
+        if hit is None or hit[0] != key:
+            idx = torch.tensor(self.buckets, dtype=torch.long,
+                               device=p.device)
+            hit = (key, p.detach().float().t()[:, idx].contiguous())
+            self.__dict__["_lut"] = hit
+        return hit[1]
+
+    def forward(self, h, meta, cache, layer_idx, shared=None):
         proj = self.qkv(h)
         fr = self._freqs(h.device) if self.rot_dims else None
         qn = self._f32("q_norm") if self.q_norm is not None else None
         kn = self._f32("k_norm") if self.k_norm is not None else None
         kpool, vpool = cache.k[layer_idx], cache.v[layer_idx]
+        v_col = self.q_cols + self.k_cols
+        rot = dict(rot_dims=self.rot_dims, freqs=fr,
+                   interleaved=self.interleaved, head_norm=self.head_norm,
+                   eps=self.eps)
         mx.norm_rope_rows(proj, self.q_cols, self.G, self.D, meta,
-                          norm_w=kn, norm_cols=self.k_cols, eps=self.eps,
-                          rot_dims=self.rot_dims, freqs=fr, pool=kpool)
-        mx.norm_rope_rows(proj, self.q_cols + self.k_cols, self.G, self.V,
-                          meta, pool=vpool)
+                          norm_w=kn, norm_cols=self.k_cols, pool=kpool, **rot)
+        first = None
+        if self.v_mix:
+            if shared is None:
+                raise ValueError("value mixing needs the step's shared "
+                                 "dictionary")
+            first = shared.get("v_first")
+            if first is None:
+                shared["v_first"] = (proj, v_col, self.v_cols)
+            elif first[2] != self.v_cols:
+                raise ValueError("value-mixing layers differ in "
+                                 "kv_heads * vdim")
+        if first is None:
+            mx.norm_rope_rows(proj, v_col, self.G, self.V, meta, pool=vpool)
+        else:
+            mx.norm_rope_rows(proj, v_col, self.G, self.V, meta, pool=vpool,
+                              mix_src=first[0], mix_col=first[1],
+                              mix_lam=self._f32("vmix").reshape(1))
         q = mx.norm_rope_rows(proj, 0, self.H, self.D, meta, norm_w=qn,
-                              norm_cols=self.q_cols, eps=self.eps,
-                              rot_dims=self.rot_dims, freqs=fr)
+                              norm_cols=self.q_cols, **rot)
         o = mx.flex_attention(
             q, kpool, vpool, meta, self.H, self.scale, window=self.window,
             sink=self.sink,
             talk=self._f32("talk") if self.talk is not None else None,
-            out_dtype=h.dtype)
+            sink_logits=self._f32("sinks") if self.sinks is not None
+            else None,
+            chunk=self.chunk, keep_first=self.keep_first,
+            dist_bias=self._dist_bias(h.device) if self.rel is not None
+            else None,
+            gate=proj if self.g_cols else None,
+            gate_col=v_col + self.v_cols, out_dtype=h.dtype)
         return self.o_proj(o)
 
 
@@ -445,6 +545,20 @@ class DenseFF(nn.Module):
 
     def forward(self, h):
         return self.down(mx.gelu(self.up(h), self.tanh_form))
+
+
+class GatedFF(nn.Module):
+    """down(gelu(gate x) * (up x)), tanh-form or exact GELU, no biases;
+    gate and up are one fused projection [gate | up]."""
+
+    def __init__(self, width: int, ff: int, tanh_form: bool = True):
+        super().__init__()
+        self.ff, self.tanh_form = int(ff), bool(tanh_form)
+        self.gate_up = TLLinear(width, 2 * ff, bias=False)
+        self.down = TLLinear(ff, width, bias=False)
+
+    def forward(self, h):
+        return self.down(mx.gelu_gate(self.gate_up(h), self.tanh_form))
 
 
 class TokenSide(nn.Module):

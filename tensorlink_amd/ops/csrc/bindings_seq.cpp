@@ -9,6 +9,8 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime.h>
 
+#include "flex_attn.hpp"
+
 extern "C" {
 void tl_postnorm_add(void* X, const void* y, const void* w, void* h,
                      int64_t rows, int W, float eps, int one_plus, int is_f32,
@@ -16,6 +18,11 @@ void tl_postnorm_add(void* X, const void* y, const void* w, void* h,
 void tl_rms_scale(const void* x, const void* w, const void* gate, int ldg,
                   int gate_col, void* out, int64_t rows, int N, float eps,
                   int one_plus, int is_f32, hipStream_t stream);
+void tl_add_rms(void* X, const void* y, const void* w, void* h, int64_t rows,
+                int W, float eps, float x_scale, int is_f32,
+                hipStream_t stream);
+void tl_gelu_gate(const void* p, void* out, int64_t rows, int N,
+                  int tanh_form, int is_f32, hipStream_t stream);
 void tl_gelu(const void* x, void* out, int64_t n, int N, int tanh_form,
              const void* table, int ldt, int table_col, const void* tokens,
              int is_f32, hipStream_t stream);
@@ -25,7 +32,10 @@ void tl_norm_rope_rows(const void* src, int ld, int col, int n_heads,
                        float eps, int rot_off, int rot_dims,
                        const void* freqs, const void* tok_seq,
                        const void* tok_pos, const void* table, int P, int T,
-                       void* out, void* pool, int is_f32, hipStream_t stream);
+                       void* out, void* pool, int is_f32, int head_norm,
+                       int interleaved, float rot_mult, const void* mix_src,
+                       int mix_ld, int mix_col, const void* mix_lam,
+                       hipStream_t stream);
 int tl_flex_attn_heads_per_block(int H, int G, int DK, int V, int has_talk);
 int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       int vld, const void* tok_seq, const void* tok_pos,
@@ -33,7 +43,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
                       int pool_f32, int hb_max, float softcap,
-                      const void* sinks, hipStream_t stream);
+                      const void* sinks, TlFlexExtra ex, hipStream_t stream);
 int tl_flex_attn_tiles_ok(int H, int G, int KG, int DK, int V);
 void tl_stage_queries(const void* q, const void* talk, void* out, int T,
                       int H, int G, int DK, hipStream_t stream);
@@ -42,7 +52,7 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                        const void* table, int P, void* out, int out_f32,
                        int H, int G, int KG, int DK, int V, float scale,
                        int window, int sink, float softcap, const void* sinks,
-                       hipStream_t stream);
+                       TlFlexExtra ex, hipStream_t stream);
 int tl_lightning_scan(const void* proj, int ld, int q_off, int k_off,
                       int v_off, const void* decay, void* S, const void* cu,
                       const void* slots, const void* pos0, void* out, int B,
@@ -130,6 +140,38 @@ Tensor rms_scale(Tensor x, Tensor w, double eps, bool one_plus,
   return out;
 }
 
+// X (*= x_scale) += y; returns rms(X) * w in the serving dtype
+Tensor add_rms(Tensor X, c10::optional<Tensor> y, Tensor w, double eps,
+               double x_scale, bool out_f32) {
+  SEQ_F32(X);
+  SEQ_F32(w);
+  TORCH_CHECK(X.dim() == 2 && w.numel() == X.size(1),
+              "X must be [T, W], the norm weight [W]");
+  if (y.has_value()) {
+    SEQ_IN(y.value());
+    TORCH_CHECK(y->sizes() == X.sizes(), "y must be [T, W]");
+    TORCH_CHECK(act_is_f32(y.value()) == (out_f32 ? 1 : 0),
+                "y / output dtype mismatch");
+  }
+  auto h = torch::empty(
+      X.sizes(), X.options().dtype(out_f32 ? torch::kFloat : torch::kBFloat16));
+  tl_add_rms(X.data_ptr(), y.has_value() ? y->data_ptr() : nullptr,
+             w.data_ptr(), h.data_ptr(), X.size(0), (int)X.size(1), (float)eps,
+             (float)x_scale, out_f32 ? 1 : 0, seq_stream());
+  return h;
+}
+
+// gelu(p[:, :N]) * p[:, N:] for p [T, 2N]
+Tensor gelu_gate(Tensor p, bool tanh_form) {
+  SEQ_IN(p);
+  TORCH_CHECK(p.dim() == 2 && p.size(1) % 2 == 0, "p must be [T, 2N]");
+  const int64_t N = p.size(1) / 2;
+  auto out = torch::empty({p.size(0), N}, p.options());
+  tl_gelu_gate(p.data_ptr(), out.data_ptr(), p.size(0), (int)N,
+               tanh_form ? 1 : 0, act_is_f32(p), seq_stream());
+  return out;
+}
+
 Tensor gelu_mul(Tensor x, bool tanh_form, c10::optional<Tensor> table,
                 c10::optional<Tensor> tokens, int64_t table_col) {
   SEQ_IN(x);
@@ -166,7 +208,10 @@ void norm_rope_rows(Tensor src, int64_t col, int64_t n_heads,
                     int64_t norm_cols, double eps, int64_t rot_off,
                     int64_t rot_dims, c10::optional<Tensor> freqs,
                     Tensor tok_seq, Tensor tok_pos, Tensor table,
-                    c10::optional<Tensor> out, c10::optional<Tensor> pool) {
+                    c10::optional<Tensor> out, c10::optional<Tensor> pool,
+                    bool head_norm, bool interleaved, double rot_mult,
+                    c10::optional<Tensor> mix_src, int64_t mix_col,
+                    c10::optional<Tensor> mix_lam) {
   SEQ_IN(src);
   SEQ_I32(tok_seq);
   SEQ_I32(tok_pos);
@@ -177,11 +222,27 @@ void norm_rope_rows(Tensor src, int64_t col, int64_t n_heads,
   TORCH_CHECK(col >= 0 && col + N <= ld, "columns out of range");
   TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T,
               "ragged metadata");
-  if (norm_w.has_value()) {
+  if (norm_w.has_value() && head_norm) {
+    SEQ_F32(norm_w.value());
+    TORCH_CHECK(norm_w->numel() == head_dim && n_heads <= 512,
+                "a per-head norm has one weight [head_dim] (<= 512 heads)");
+  } else if (norm_w.has_value()) {
     SEQ_F32(norm_w.value());
     TORCH_CHECK(norm_cols > 0 && norm_cols <= N &&
                     norm_w->numel() == norm_cols,
                 "norm weight must cover the normed columns");
+  }
+  int mix_ld = 0;
+  if (mix_src.has_value()) {
+    SEQ_IN(mix_src.value());
+    TORCH_CHECK(mix_lam.has_value(), "blending needs its weight");
+    SEQ_F32(mix_lam.value());
+    TORCH_CHECK(mix_src->scalar_type() == src.scalar_type() &&
+                    mix_src->dim() == 2 && mix_src->size(0) == T &&
+                    mix_col >= 0 && mix_col + N <= mix_src->size(1) &&
+                    mix_lam->numel() == 1,
+                "blend source must be [T, >= mix_col + N] of src's dtype");
+    mix_ld = (int)mix_src->size(1);
   }
   if (rot_dims > 0) {
     TORCH_CHECK(freqs.has_value(), "rotation needs frequencies");
@@ -191,7 +252,7 @@ void norm_rope_rows(Tensor src, int64_t col, int64_t n_heads,
                     rot_off >= 0 && rot_off + rot_dims <= head_dim,
                 "frequencies must be float64 [rot_dims / 2]");
     // a rotated pair must be normed alike
-    TORCH_CHECK(!norm_w.has_value() || norm_cols == N ||
+    TORCH_CHECK(!norm_w.has_value() || head_norm || norm_cols == N ||
                     (n_heads == 1 && (norm_cols <= rot_off)),
                 "the norm range may not cut a rotated pair");
   }
@@ -216,7 +277,43 @@ void norm_rope_rows(Tensor src, int64_t col, int64_t n_heads,
       tok_pos.data_ptr(), table.data_ptr(), (int)table.size(1), (int)T,
       out.has_value() ? out->data_ptr() : nullptr,
       pool.has_value() ? pool->data_ptr() : nullptr, act_is_f32(src),
+      head_norm ? 1 : 0, interleaved ? 1 : 0, (float)rot_mult,
+      mix_src.has_value() ? mix_src->data_ptr() : nullptr, mix_ld,
+      (int)mix_col, mix_lam.has_value() ? mix_lam->data_ptr() : nullptr,
       seq_stream());
+}
+
+// checked options of the flexible attention beyond window / sink / cap
+TlFlexExtra flex_extra(int64_t T, int64_t H, int64_t V, int64_t window,
+                       int64_t chunk, int64_t keep,
+                       const c10::optional<Tensor>& bias,
+                       const c10::optional<Tensor>& gate, int64_t gate_col,
+                       bool gate_heads) {
+  TlFlexExtra ex{};
+  TORCH_CHECK(chunk >= 0 && keep >= 0 && !(chunk > 0 && window > 0),
+              "a chunked mask has no window");
+  ex.chunk = (int)chunk;
+  ex.keep = (int)keep;
+  if (bias.has_value()) {
+    SEQ_F32(bias.value());
+    TORCH_CHECK(bias->dim() == 2 && bias->size(0) == H && bias->size(1) >= 1,
+                "distance bias must be [H, n]");
+    ex.bias = (const float*)bias->data_ptr();
+    ex.nb = (int)bias->size(1);
+  }
+  if (gate.has_value()) {
+    SEQ_IN(gate.value());
+    const int64_t n = gate_heads ? H : H * V;
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == T && gate_col >= 0 &&
+                    gate_col + n <= gate->size(1),
+                "gate columns out of range");
+    ex.gate = gate->data_ptr();
+    ex.gate_ld = (int)gate->size(1);
+    ex.gate_col = (int)gate_col;
+    ex.gate_heads = gate_heads ? 1 : 0;
+    ex.gate_f32 = act_is_f32(gate.value());
+  }
+  return ex;
 }
 
 Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
@@ -224,7 +321,10 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
                       c10::optional<Tensor> talk, int64_t H, double scale,
                       int64_t window, bool sink, int64_t V, bool out_f32,
                       int64_t n_split, int64_t hb_max, double softcap,
-                      c10::optional<Tensor> sinks) {
+                      c10::optional<Tensor> sinks, int64_t chunk,
+                      int64_t keep, c10::optional<Tensor> bias,
+                      c10::optional<Tensor> gate, int64_t gate_col,
+                      bool gate_heads) {
   if (sinks.has_value()) {
     SEQ_F32(sinks.value());
     TORCH_CHECK(sinks->numel() == H && sink, "sink logits must be [H]");
@@ -262,6 +362,8 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
   }
   TORCH_CHECK(window >= 0 && n_split >= 1 && n_split <= 64,
               "window / n_split out of range");
+  const TlFlexExtra ex =
+      flex_extra(T, H, V, window, chunk, keep, bias, gate, gate_col, gate_heads);
   TORCH_CHECK(tl_flex_attn_heads_per_block((int)H, G, DK, (int)V,
                                            talk.has_value() ? 1 : 0) > 0,
               "flex_attn_rows: shape outside the kernel's range (value size "
@@ -281,7 +383,7 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
       out_f32 ? 1 : 0, n_split > 1 ? part.data_ptr() : nullptr, (int)n_split,
       (int)T, (int)H, G, DK, (int)V, (float)scale, (int)window, sink ? 1 : 0,
       pool_f32, (int)std::max<int64_t>(1, hb_max), (float)softcap,
-      sinks.has_value() ? sinks->data_ptr() : nullptr, seq_stream());
+      sinks.has_value() ? sinks->data_ptr() : nullptr, ex, seq_stream());
   TORCH_CHECK(rc == 0, "flex_attn_rows: launch refused");
   return out;
 }
@@ -298,7 +400,10 @@ Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
                        Tensor tiles, Tensor table,
                        c10::optional<Tensor> talk, int64_t H, double scale,
                        int64_t window, bool sink, int64_t V, bool out_f32,
-                       double softcap, c10::optional<Tensor> sinks) {
+                       double softcap, c10::optional<Tensor> sinks,
+                       int64_t chunk, int64_t keep,
+                       c10::optional<Tensor> bias, c10::optional<Tensor> gate,
+                       int64_t gate_col, bool gate_heads) {
   if (sinks.has_value()) {
     SEQ_F32(sinks.value());
     TORCH_CHECK(sinks->numel() == H && sink, "sink logits must be [H]");
@@ -337,6 +442,8 @@ Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
   const int KG = talk.has_value() ? G : 1;
   TORCH_CHECK(tl_flex_attn_tiles_ok((int)H, G, KG, DK, (int)V),
               "flex_attn_tiles: shape outside the kernel's range");
+  const TlFlexExtra ex =
+      flex_extra(T, H, V, window, chunk, keep, bias, gate, gate_col, gate_heads);
   auto qs = torch::empty({T, H * KG * DK},
                          q.options().dtype(torch::kBFloat16));
   auto out = torch::empty(
@@ -351,7 +458,7 @@ Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
       (int)tiles.size(0), table.data_ptr(), (int)table.size(1),
       out.data_ptr(), out_f32 ? 1 : 0, (int)H, G, KG, DK, (int)V,
       (float)scale, (int)window, sink ? 1 : 0, (float)softcap,
-      sinks.has_value() ? sinks->data_ptr() : nullptr, seq_stream());
+      sinks.has_value() ? sinks->data_ptr() : nullptr, ex, seq_stream());
   TORCH_CHECK(rc == 0, "flex_attn_tiles: launch refused");
   return out;
 }
@@ -465,6 +572,9 @@ void register_seq_ops(pybind11::module& mod) {
   mod.def("postnorm_add", &postnorm_add,
           "X += y / rms(y) * g on the fp32 residual; returns the cast copy");
   mod.def("rms_scale", &rms_scale, "x / rms(x) * g [* sigmoid(gate)]");
+  mod.def("add_rms", &add_rms,
+          "X += y on the fp32 residual; returns rms(X) * w (pre-norm)");
+  mod.def("gelu_gate", &gelu_gate, "gelu(gate) * up on a fused projection");
   mod.def("gelu_mul", &gelu_mul,
           "GELU (erf or tanh form) times an optional gathered table slice");
   mod.def("soft_cap_", &soft_cap_, "cap * tanh(z / cap) in place");

@@ -19,12 +19,18 @@
 // between the mixed query [sum_{g in c} T[h,g] q_g]_c and the G key heads'
 // rows side by side: the block stages mixed queries and then works as if
 // the key were G times as wide.
+// Further options (TlFlexExtra): keys of the query's own chunk only, a kept
+// prefix (the first positions stay visible beyond the window: the block
+// walks the prefix tiles, then the window's), a learned distance bias from
+// a per-head table indexed by i - j, and a sigmoid output gate per column
+// or per head applied where the row is written.
 // With few rows over long ranges the keys are also split over blockIdx.z
 // and a merge kernel finishes the rows. It is exact for any query position,
 // so it serves prompt portions and decoding alike; scores, weights and
 // sums are fp32.
 
 #include "common.hpp"
+#include "flex_attn.hpp"
 
 #include <cstdlib>
 
@@ -34,6 +40,7 @@ constexpr int PAGE = 128;
 static_assert(PAGE % WAVE_SIZE == 0, "a key tile must not straddle pages");
 constexpr int NWAVE = 4;
 constexpr int BLOCK = NWAVE * WAVE_SIZE;
+constexpr int MAX_NORM_HEADS = 512;   // heads of a per-head normed row
 
 template <typename T> DEVINLINE float ldv(const T* p);
 template <> DEVINLINE float ldv<float>(const float* p) { return *p; }
@@ -50,13 +57,29 @@ __global__ __launch_bounds__(BLOCK) void norm_rope_rows_kernel(
     int rot_dims, const double* __restrict__ freqs,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
     const int* __restrict__ table, int P, float* __restrict__ out,
-    T* __restrict__ pool) {
+    T* __restrict__ pool, int head_norm, int interleaved, float rot_mult,
+    const T* __restrict__ mix_src, int mix_ld, int mix_col,
+    const float* __restrict__ mix_lam) {
   __shared__ float red[NWAVE];
+  __shared__ float head_rn[MAX_NORM_HEADS];
   const int t = blockIdx.x;
   const int N = n_heads * head_dim;
   const T* row = src + (int64_t)t * ld + col;
   float rn = 1.f;
-  if (norm_w) {
+  if (norm_w && head_norm) {
+    // one statistic per head, the weight [head_dim] shared by the heads
+    const int lane = threadIdx.x & (WAVE_SIZE - 1);
+    for (int hd = threadIdx.x / WAVE_SIZE; hd < n_heads; hd += NWAVE) {
+      float ss = 0.f;
+      for (int e = lane; e < head_dim; e += WAVE_SIZE) {
+        const float v = ldv<T>(row + hd * head_dim + e);
+        ss += v * v;
+      }
+      ss = wave_reduce_sum(ss);
+      if (lane == 0) head_rn[hd] = 1.0f / sqrtf(ss / (float)head_dim + eps);
+    }
+    __syncthreads();
+  } else if (norm_w) {
     float ss = 0.f;
     for (int c = threadIdx.x; c < norm_cols; c += BLOCK) {
       const float v = ldv<T>(row + c);
@@ -72,21 +95,36 @@ __global__ __launch_bounds__(BLOCK) void norm_rope_rows_kernel(
     const int page = table[(int64_t)tok_seq[t] * P + pos / PAGE];
     prow = (int64_t)page * n_heads * PAGE + (pos % PAGE);
   }
+  const float lam = mix_src ? mix_lam[0] : 0.f;
   for (int c = threadIdx.x; c < N; c += BLOCK) {
     const int hd = c / head_dim, e = c - hd * head_dim;
     float x = ldv<T>(row + c);
-    if (norm_w && c < norm_cols) x = x * rn * norm_w[c];
+    if (norm_w) {
+      if (head_norm) x = x * head_rn[hd] * norm_w[e];
+      else if (c < norm_cols) x = x * rn * norm_w[c];
+    }
     const int r = e - rot_off;
     if (r >= 0 && r < rot_dims) {
-      const int i = r < half ? r : r - half;
-      const int cp = r < half ? c + half : c - half;   // the pair's other
+      // the pair's first member: r < half (halves) or r even (interleaved)
+      const bool is_u = interleaved ? (r & 1) == 0 : r < half;
+      const int i = interleaved ? r >> 1 : (r < half ? r : r - half);
+      const int step = interleaved ? 1 : half;
+      const int cp = is_u ? c + step : c - step;       // the pair's other
       float y = ldv<T>(row + cp);
-      if (norm_w && cp < norm_cols) y = y * rn * norm_w[cp];
+      if (norm_w) {
+        if (head_norm) y = y * head_rn[hd] * norm_w[cp - hd * head_dim];
+        else if (cp < norm_cols) y = y * rn * norm_w[cp];
+      }
       const double ang = (double)pos * freqs[i];
-      const float cs = (float)cos(ang), sn = (float)sin(ang);
+      const float cs = (float)cos(ang) * rot_mult;
+      const float sn = (float)sin(ang) * rot_mult;
       // (u, v) -> (u cos - v sin, v cos + u sin); x is u or v
-      x = r < half ? x * cs - y * sn : x * cs + y * sn;
+      x = is_u ? x * cs - y * sn : x * cs + y * sn;
     }
+    // blend with the same token's row of another projection
+    if (mix_src)
+      x = (1.f - lam) * x +
+          lam * ldv<T>(mix_src + (int64_t)t * mix_ld + mix_col + c);
     if (pool)
       stv<T>(pool + (prow + (int64_t)hd * PAGE) * head_dim + e, x);
     else
@@ -95,6 +133,17 @@ __global__ __launch_bounds__(BLOCK) void norm_rope_rows_kernel(
 }
 
 // -------------------------------------------------------------- attention
+// sigmoid of the output gate of column c of head h of token t; 1 without
+DEVINLINE float out_gate(const TlFlexExtra& ex, int64_t t, int h, int V,
+                         int c) {
+  if (!ex.gate) return 1.f;
+  const int64_t i =
+      t * ex.gate_ld + ex.gate_col + (ex.gate_heads ? h : h * V + c);
+  const float g = ex.gate_f32 ? ((const float*)ex.gate)[i]
+                              : bf2f(((const bf16*)ex.gate)[i]);
+  return 1.f / (1.f + expf(-g));
+}
+
 // part row (key split z of token t, head h): m, l, acc[V]
 template <typename TK, int HB, int VR, bool TALK>
 __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
@@ -103,7 +152,8 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
     const int* __restrict__ tok_pos, const int* __restrict__ table, int P,
     const float* __restrict__ talk, void* __restrict__ out, int out_f32,
     float* __restrict__ part, int H, int G, int DK, int V, float scale,
-    int window, int sink, float softcap, const float* __restrict__ sinks) {
+    int window, int sink, float softcap, const float* __restrict__ sinks,
+    TlFlexExtra ex) {
   extern __shared__ float lds[];
   const int t = blockIdx.x, h0 = blockIdx.y * HB;
   const int ns = gridDim.z, z = blockIdx.z;
@@ -148,13 +198,19 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
 #pragma unroll
     for (int r = 0; r < AC; ++r) a[b][r] = 0.f;
   }
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = tl_flex_lo(pos, window, ex.chunk);
   const int first = (lo / WAVE_SIZE) * WAVE_SIZE;
+  // kept prefix [0, kp) below the main range [lo, pos]: its tiles come first
+  const int kp = min(ex.keep, lo);
+  const int n_pre = (kp + WAVE_SIZE - 1) / WAVE_SIZE;
   const bool vec8 = sizeof(TK) == 2 && (DK % 8) == 0;
-  for (int j0 = first + (z * NWAVE + wave) * WAVE_SIZE; j0 <= pos;
-       j0 += ns * NWAVE * WAVE_SIZE) {
+  for (int it = z * NWAVE + wave;; it += ns * NWAVE) {
+    const bool pre = it < n_pre;
+    const int j0 = pre ? it * WAVE_SIZE : first + (it - n_pre) * WAVE_SIZE;
+    if (j0 > pos) break;
+    const int rlo = pre ? 0 : lo, rhi = pre ? kp - 1 : pos;
     const int j = j0 + lane;
-    const bool valid = j >= lo && j <= pos;
+    const bool valid = j >= rlo && j <= rhi;
     // a 64-key tile lies inside ONE 128-position page
     const int64_t page_row = (int64_t)tab[j0 / PAGE] * G * PAGE + (j0 % PAGE);
     float s[HB];
@@ -187,9 +243,13 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       }
     }
     float p[HB];
+    const float* brow =
+        ex.bias ? ex.bias + (int64_t)h0 * ex.nb + min(max(pos - j, 0), ex.nb - 1)
+                : nullptr;
 #pragma unroll
     for (int b = 0; b < HB; ++b) {
-      const float sc = softcap > 0.f ? softcap * tanhf(s[b] / softcap) : s[b];
+      float sc = softcap > 0.f ? softcap * tanhf(s[b] / softcap) : s[b];
+      if (brow && valid) sc += brow[(int64_t)b * ex.nb];
       const float sv = valid ? sc : -INFINITY;
       const float nm = fmaxf(m[b], wave_reduce_max(sv));
       // nm is finite: every tile of the loop holds at least one valid key
@@ -200,7 +260,7 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
 #pragma unroll
       for (int r = 0; r < AC; ++r) a[b][r] *= c;
     }
-    const int jb = max(0, lo - j0), je = min(WAVE_SIZE, pos + 1 - j0);
+    const int jb = max(0, rlo - j0), je = min(WAVE_SIZE, rhi + 1 - j0);
     const TK* vtile = vpool + (page_row + (int64_t)g0 * PAGE) * vld;
     if constexpr (VR == 0) {
       const int CPR = V >> 3, KGR = WAVE_SIZE / CPR;
@@ -317,10 +377,11 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       float A = 0.f;
       for (int w = 0; w < NWAVE; ++w) A += f[w] * accs[(w * HB + b) * V + c];
       const int64_t o = ((int64_t)t * H + h0 + b) * V + c;
+      const float r = A / L * out_gate(ex, t, h0 + b, V, c);
       if (out_f32)
-        ((float*)out)[o] = A / L;
+        ((float*)out)[o] = r;
       else
-        ((bf16*)out)[o] = f2bf(A / L);
+        ((bf16*)out)[o] = f2bf(r);
     }
   }
 }
@@ -328,7 +389,8 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
 // one block per (token, head): merge the key splits
 __global__ __launch_bounds__(BLOCK) void flex_attn_merge_kernel(
     const float* __restrict__ part, void* __restrict__ out, int out_f32,
-    int ns, int V, int sink, int H, const float* __restrict__ sinks) {
+    int ns, int V, int sink, int H, const float* __restrict__ sinks,
+    TlFlexExtra ex) {
   const int64_t row = blockIdx.x;
   const float* pr = part + row * ns * (2 + V);
   float M = -INFINITY;
@@ -346,10 +408,11 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_merge_kernel(
       const float mz = pr[z * (2 + V)];
       A += (mz == -INFINITY ? 0.f : expf(mz - M)) * pr[z * (2 + V) + 2 + c];
     }
+    const float r = A / L * out_gate(ex, row / H, (int)(row % H), V, c);
     if (out_f32)
-      ((float*)out)[row * V + c] = A / L;
+      ((float*)out)[row * V + c] = r;
     else
-      ((bf16*)out)[row * V + c] = f2bf(A / L);
+      ((bf16*)out)[row * V + c] = f2bf(r);
   }
 }
 
@@ -359,17 +422,18 @@ void launch_rows(bool has_talk, dim3 grid, size_t smem, hipStream_t stream,
                  const int* tok_seq, const int* tok_pos, const int* table,
                  int P, const float* talk, void* out, int out_f32,
                  float* part, int H, int G, int DK, int V, float scale,
-                 int window, int sink, float softcap, const float* sinks) {
+                 int window, int sink, float softcap, const float* sinks,
+                 const TlFlexExtra& ex) {
   if (has_talk)
     hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, true>), grid,
                        dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
                        tok_seq, tok_pos, table, P, talk, out, out_f32, part,
-                       H, G, DK, V, scale, window, sink, softcap, sinks);
+                       H, G, DK, V, scale, window, sink, softcap, sinks, ex);
   else
     hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, false>), grid,
                        dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
                        tok_seq, tok_pos, table, P, talk, out, out_f32, part,
-                       H, G, DK, V, scale, window, sink, softcap, sinks);
+                       H, G, DK, V, scale, window, sink, softcap, sinks, ex);
 }
 
 size_t rows_smem(bool has_talk, int hb, int G, int DK, int V) {
@@ -386,7 +450,9 @@ void tl_norm_rope_rows(const void* src, int ld, int col, int n_heads,
                        float eps, int rot_off, int rot_dims,
                        const void* freqs, const void* tok_seq,
                        const void* tok_pos, const void* table, int P, int T,
-                       void* out, void* pool, int is_f32,
+                       void* out, void* pool, int is_f32, int head_norm,
+                       int interleaved, float rot_mult, const void* mix_src,
+                       int mix_ld, int mix_col, const void* mix_lam,
                        hipStream_t stream) {
   if (T <= 0) return;
   dim3 grid(T), block(BLOCK);
@@ -396,14 +462,18 @@ void tl_norm_rope_rows(const void* src, int ld, int col, int n_heads,
                        (const float*)norm_w, norm_cols, eps, rot_off,
                        rot_dims, (const double*)freqs, (const int*)tok_seq,
                        (const int*)tok_pos, (const int*)table, P,
-                       (float*)out, (float*)pool);
+                       (float*)out, (float*)pool, head_norm, interleaved,
+                       rot_mult, (const float*)mix_src, mix_ld, mix_col,
+                       (const float*)mix_lam);
   else
     hipLaunchKernelGGL(norm_rope_rows_kernel<bf16>, grid, block, 0, stream,
                        (const bf16*)src, ld, col, n_heads, head_dim,
                        (const float*)norm_w, norm_cols, eps, rot_off,
                        rot_dims, (const double*)freqs, (const int*)tok_seq,
                        (const int*)tok_pos, (const int*)table, P,
-                       (float*)out, (bf16*)pool);
+                       (float*)out, (bf16*)pool, head_norm, interleaved,
+                       rot_mult, (const bf16*)mix_src, mix_ld, mix_col,
+                       (const float*)mix_lam);
 }
 
 // heads per block for a shape: the largest of 8, 4, 2, 1 that divides the
@@ -434,7 +504,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
                       int pool_f32, int hb_max, float softcap,
-                      const void* sinks, hipStream_t stream) {
+                      const void* sinks, TlFlexExtra ex, hipStream_t stream) {
   if (T <= 0) return 0;
   const bool has_talk = talk != nullptr;
   static const bool no_vec = getenv("TL_NO_VEC_VALUES") != nullptr;
@@ -449,7 +519,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                             (const int*)tok_seq, (const int*)tok_pos,        \
                             (const int*)table, P, (const float*)talk, out,   \
                             out_f32, (float*)part, H, G, DK, V, scale,       \
-                            window, sink, softcap, (const float*)sinks)
+                            window, sink, softcap, (const float*)sinks, ex)
 #define TL_FA_V(TT, HBB)                     \
   if (vr <= 1) TL_FA(TT, HBB, 1);            \
   else if (vr <= 2) TL_FA(TT, HBB, 2);       \
@@ -480,7 +550,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
   if (ns > 1)
     hipLaunchKernelGGL(flex_attn_merge_kernel, dim3(T * H), dim3(BLOCK), 0,
                        stream, (const float*)part, out, out_f32, ns, V, sink, H,
-                       (const float*)sinks);
+                       (const float*)sinks, ex);
   return 0;
 }
 

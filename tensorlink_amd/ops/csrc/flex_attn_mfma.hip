@@ -20,10 +20,15 @@
 // tl_stage_queries builds those mixed queries (or plain copies) in bf16
 // from the fp32 normed/rotated queries; the tile kernel then only sees a
 // query of KG*DK columns that meets KG key heads.
+// Further options (TlFlexExtra): keys of the query's own chunk only, a kept
+// prefix (its key tiles are walked before the window's), a learned distance
+// bias from a per-head table indexed by i - j, a sigmoid output gate per
+// column or per head applied to the normalised row.
 // Scores, softmax statistics and accumulators are fp32; P is rounded to
 // bf16 only as the MFMA operand.
 
 #include "common.hpp"
+#include "flex_attn.hpp"
 
 namespace {
 
@@ -90,7 +95,8 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
     const int* __restrict__ tiles,   // [n][4]: seq, first token, count, pos
     const int* __restrict__ table, int P, void* __restrict__ out,
     int out_f32, int H, int G, int KG, int DK, int V, float scale,
-    int window, int sink, float softcap, const float* __restrict__ sinks) {
+    int window, int sink, float softcap, const float* __restrict__ sinks,
+    TlFlexExtra ex) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   bf16* vt_lds = reinterpret_cast<bf16*>(smem_raw);     // [V][VLD]
 
@@ -117,9 +123,16 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
   const int wave_first = p0 + min(wave * 16, n - 1);
   const int wave_last = p0 + min(wave * 16 + 15, n - 1);
   const bool wave_on = wave * 16 < n;
-  const int k_begin =
-      window > 0 ? (max(0, p0 - window + 1) / KT) * KT : 0;
-  const int wave_old = window > 0 ? wave_first - window + 1 : 0;
+  // lo() grows with the position: the block's oldest key is its first
+  // query's, a wave's oldest its first query's
+  const int k_begin = (tl_flex_lo(p0, window, ex.chunk) / KT) * KT;
+  const int wave_old = tl_flex_lo(wave_first, window, ex.chunk);
+  const int lo_q = tl_flex_lo(qpos, window, ex.chunk);
+  const int keep = ex.keep;
+  // kept prefix below the main range: rounds [0, n_pre) walk its tiles
+  const int n_pre = (min(keep, k_begin) + KT - 1) / KT;
+  const int n_round = n_pre + (k_end - k_begin + KT - 1) / KT;
+  const float* brow = ex.bias ? ex.bias + (int64_t)h * ex.nb : nullptr;
 
   bf16x8_t qf[QCMAX];
 #pragma unroll
@@ -141,7 +154,8 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
 
   const int vchunks = V / 8;                // 16-byte chunks per value row
-  for (int k0 = k_begin; k0 < k_end; k0 += KT) {
+  for (int rd = 0; rd < n_round; ++rd) {
+    const int k0 = rd < n_pre ? rd * KT : k_begin + (rd - n_pre) * KT;
     __syncthreads();                        // previous round's reads done
     // lane -> key fastest: the 2-byte transposed stores of a wave then
     // fall into consecutive LDS words instead of a few banks
@@ -157,14 +171,16 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
     }
     __syncthreads();
     // wave-uniform skips: keys after the wave's last query, or older than
-    // the window of its first
-    if (!wave_on || k0 > wave_last || k0 + KT - 1 < wave_old) continue;
+    // the range of its first and not of the kept prefix
+    if (!wave_on || k0 > wave_last ||
+        (k0 + KT - 1 < wave_old && k0 >= keep))
+      continue;
 
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int kb = k0 + sub * 32;
       if (kb > wave_last) break;
-      if (kb + 31 < wave_old) continue;
+      if (kb + 31 < wave_old && kb >= keep) continue;
       // ---- S^T for two 16-key tiles
       f32x4 st[2];
 #pragma unroll
@@ -195,10 +211,10 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = kb + t16 * 16 + quad * 4 + r;
-          const bool ok =
-              key <= qpos && (window <= 0 || key > qpos - window);
+          const bool ok = key <= qpos && (key >= lo_q || key < keep);
           float s = st[t16][r] * scale;
           if (softcap > 0.f) s = softcap * fast_tanh(s * inv_cap);
+          if (brow) s += brow[min(max(qpos - key, 0), ex.nb - 1)];
           s = ok ? s : -INFINITY;
           sv[t16 * 4 + r] = s;
           mx = fmaxf(mx, s);
@@ -259,14 +275,27 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
 #pragma unroll
     for (int vt = 0; vt < VTMAX; ++vt)
       if (vt < nvt) {
+        float g4[4] = {1.f, 1.f, 1.f, 1.f};
+        if (ex.gate) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int64_t gi =
+                (int64_t)tok * ex.gate_ld + ex.gate_col +
+                (ex.gate_heads ? h : h * V + vt * 16 + quad * 4 + r);
+            const float g = ex.gate_f32 ? ((const float*)ex.gate)[gi]
+                                        : bf2f(((const bf16*)ex.gate)[gi]);
+            g4[r] = 1.f / (1.f + __expf(-g));
+          }
+        }
         if (out_f32) {
           float* orow = (float*)out + o0 + vt * 16 + quad * 4;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) orow[r] = acc[vt][r] * inv;
+          for (int r = 0; r < 4; ++r) orow[r] = acc[vt][r] * inv * g4[r];
         } else {
           bf16x4_t o4;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o4[r] = (__bf16)(acc[vt][r] * inv);
+          for (int r = 0; r < 4; ++r)
+            o4[r] = (__bf16)(acc[vt][r] * inv * g4[r]);
           *reinterpret_cast<bf16x4_t*>((bf16*)out + o0 + vt * 16 + quad * 4) =
               o4;
         }
@@ -300,7 +329,7 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                        const void* table, int P, void* out, int out_f32,
                        int H, int G, int KG, int DK, int V, float scale,
                        int window, int sink, float softcap, const void* sinks,
-                       hipStream_t stream) {
+                       TlFlexExtra ex, hipStream_t stream) {
   if (!tl_flex_attn_tiles_ok(H, G, KG, DK, V) || vld % 8 != 0 ||
       n_tiles <= 0)
     return 1;
@@ -312,7 +341,7 @@ int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
                      stream, (const bf16*)q, (const bf16*)kpool,             \
                      (const bf16*)vpool, vld, (const int*)tiles,             \
                      (const int*)table, P, out, out_f32, H, G, KG, DK, V,    \
-                     scale, window, sink, softcap, (const float*)sinks)
+                     scale, window, sink, softcap, (const float*)sinks, ex)
 #define TL_FT_V(QCC)                          \
   if (nvt <= 4) TL_FT_LAUNCH(QCC, 4);         \
   else if (nvt <= 8) TL_FT_LAUNCH(QCC, 8);    \

@@ -9,6 +9,12 @@
 // read-out norm of a linear-attention mixer with its sigmoid gate), tl_gelu
 // the exact or tanh-form GELU with an optional gathered per-token factor,
 // tl_soft_cap the logit cap. Statistics and activations are fp32.
+//
+// Pre-norm layers use tl_add_rms: the previous sublayer's output is added
+// to the fp32 residual and the NEXT sublayer's input, rms(X) * w, is written
+// in the serving dtype by the same kernel (X <- X + y;  h = X / rms(X) * w).
+// tl_gelu_gate is the gated feed-forward's activation on a fused [gate | up]
+// projection: gelu(gate) * up.
 
 #include "common.hpp"
 
@@ -23,6 +29,13 @@ template <> DEVINLINE float ldf<bf16>(const bf16* p, int64_t i) { return bf2f(p[
 template <typename T> DEVINLINE void stf(T* p, int64_t i, float v);
 template <> DEVINLINE void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
 template <> DEVINLINE void stf<bf16>(bf16* p, int64_t i, float v) { p[i] = f2bf(v); }
+
+DEVINLINE float gelu_f(float z, int tanh_form) {
+  if (tanh_form)
+    return 0.5f * z *
+           (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+}
 
 // one block per row
 template <typename T>
@@ -49,6 +62,60 @@ __global__ __launch_bounds__(BLOCK) void postnorm_add_kernel(
   }
 }
 
+// X += y (if given); h = X / rms(X) * w in the serving dtype
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void add_rms_kernel(
+    float* __restrict__ X, const T* __restrict__ y,
+    const float* __restrict__ w, T* __restrict__ h, int W, float eps,
+    float x_scale) {
+  __shared__ float red[NW];
+  const int64_t row = blockIdx.x;
+  float* xr = X + row * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += BLOCK) {
+    float v = xr[c] * x_scale;
+    if (y) v += ldf<T>(y, row * W + c);
+    if (y || x_scale != 1.f) xr[c] = v;
+    ss += v * v;
+  }
+  const float tot = block_reduce_sum<NW>(ss, red);
+  const float rn = 1.0f / sqrtf(tot / (float)W + eps);
+  // a thread reads back only what it wrote itself
+  for (int c = threadIdx.x; c < W; c += BLOCK)
+    stf<T>(h, row * W + c, xr[c] * rn * w[c]);
+}
+
+// out[r][c] = gelu(p[r][c]) * p[r][N + c] on rows of 2N columns
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void gelu_gate_kernel(
+    const T* __restrict__ p, T* __restrict__ out, int64_t n, int N,
+    int tanh_form) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * BLOCK) {
+    const int64_t r = i / N;
+    const int c = (int)(i - r * N);
+    const T* row = p + r * 2 * N;
+    stf<T>(out, i, gelu_f(ldf<T>(row, c), tanh_form) * ldf<T>(row, N + c));
+  }
+}
+
+// bf16 rows whose half width is a multiple of 8: 16-byte loads and stores
+__global__ __launch_bounds__(BLOCK) void gelu_gate_vec8_kernel(
+    const bf16x8* __restrict__ p, bf16x8* __restrict__ out, int64_t n8,
+    int N8, int tanh_form) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * BLOCK) {
+    const int64_t r = i / N8;
+    const int c = (int)(i - r * N8);
+    const bf16x8 a = p[r * 2 * N8 + c], b = p[r * 2 * N8 + N8 + c];
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      o.v[e] = f2bf(gelu_f(bf2f(a.v[e]), tanh_form) * bf2f(b.v[e]));
+    out[i] = o;
+  }
+}
+
 // out = x / rms(x) * g [* sigmoid(gate)], x fp32 [rows, N]
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void rms_scale_kernel(
@@ -70,13 +137,6 @@ __global__ __launch_bounds__(BLOCK) void rms_scale_kernel(
     }
     stf<T>(out, row * N + c, v);
   }
-}
-
-DEVINLINE float gelu_f(float z, int tanh_form) {
-  if (tanh_form)
-    return 0.5f * z *
-           (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-  return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
 }
 
 template <typename T>
@@ -139,6 +199,40 @@ void tl_postnorm_add(void* X, const void* y, const void* w, void* h,
     hipLaunchKernelGGL(postnorm_add_kernel<bf16>, grid, block, 0, stream,
                        (float*)X, (const bf16*)y, (const float*)w, (bf16*)h,
                        W, eps, one_plus);
+}
+
+void tl_add_rms(void* X, const void* y, const void* w, void* h, int64_t rows,
+                int W, float eps, float x_scale, int is_f32,
+                hipStream_t stream) {
+  if (rows <= 0) return;
+  dim3 grid((unsigned)rows), block(BLOCK);
+  if (is_f32)
+    hipLaunchKernelGGL(add_rms_kernel<float>, grid, block, 0, stream,
+                       (float*)X, (const float*)y, (const float*)w, (float*)h,
+                       W, eps, x_scale);
+  else
+    hipLaunchKernelGGL(add_rms_kernel<bf16>, grid, block, 0, stream,
+                       (float*)X, (const bf16*)y, (const float*)w, (bf16*)h,
+                       W, eps, x_scale);
+}
+
+void tl_gelu_gate(const void* p, void* out, int64_t rows, int N,
+                  int tanh_form, int is_f32, hipStream_t stream) {
+  const int64_t n = rows * N;
+  if (n <= 0) return;
+  if (!is_f32 && N % 8 == 0) {
+    hipLaunchKernelGGL(gelu_gate_vec8_kernel, dim3(ew_grid(n / 8)),
+                       dim3(BLOCK), 0, stream, (const bf16x8*)p, (bf16x8*)out,
+                       n / 8, N / 8, tanh_form);
+    return;
+  }
+  dim3 grid(ew_grid(n)), block(BLOCK);
+  if (is_f32)
+    hipLaunchKernelGGL(gelu_gate_kernel<float>, grid, block, 0, stream,
+                       (const float*)p, (float*)out, n, N, tanh_form);
+  else
+    hipLaunchKernelGGL(gelu_gate_kernel<bf16>, grid, block, 0, stream,
+                       (const bf16*)p, (bf16*)out, n, N, tanh_form);
 }
 
 void tl_rms_scale(const void* x, const void* w, const void* gate, int ldg,

@@ -432,6 +432,37 @@ def soft_cap_(z: torch.Tensor, cap: float) -> torch.Tensor:
     return z.copy_(cap * torch.tanh(z / cap))
 
 
+def add_rms(X: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor,
+            eps: float, out_dtype=torch.float32,
+            x_scale: float = 1.0) -> torch.Tensor:
+    """Pre-norm residual step, in place on the fp32 residual X [T, W]:
+    X <- X * x_scale + y (``y`` = the previous sublayer's output, or None),
+    then returns the next sublayer's input X / rms(X) * w in ``out_dtype``.
+    Sum, statistic and scaling are fp32."""
+    assert X.dtype == torch.float32 and w.dtype == torch.float32
+    if X.is_cuda:
+        return _ext().add_rms(X, None if y is None else y.contiguous(), w,
+                              float(eps), float(x_scale),
+                              out_dtype == torch.float32)
+    if x_scale != 1.0:
+        X *= x_scale
+    if y is not None:
+        X += y.float()
+    return (_rms(X, eps) * w).to(out_dtype)
+
+
+def gelu_gate(p: torch.Tensor, tanh_form: bool = True) -> torch.Tensor:
+    """gelu(p[:, :N]) * p[:, N:] for a fused [gate | up] projection
+    p [T, 2N]; evaluated in fp32, result in p's dtype."""
+    if p.is_cuda:
+        return _ext().gelu_gate(p.contiguous(), bool(tanh_form))
+    N = p.shape[1] // 2
+    f = p.float()
+    y = torch.nn.functional.gelu(
+        f[:, :N], approximate="tanh" if tanh_form else "none") * f[:, N:]
+    return y.to(p.dtype)
+
+
 # ---------------------------------------------------------------------------
 # row preparation: RMS norm over a projection + rotate-half positions,
 # written densely (queries) or into a page pool (keys, values, latents)
@@ -448,14 +479,23 @@ def norm_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
                    meta: RaggedMeta, *, norm_w: Optional[torch.Tensor] = None,
                    norm_cols: int = 0, eps: float = 0.0, rot_off: int = 0,
                    rot_dims: int = 0, freqs: Optional[torch.Tensor] = None,
-                   pool: Optional[torch.Tensor] = None):
+                   pool: Optional[torch.Tensor] = None,
+                   head_norm: bool = False, interleaved: bool = False,
+                   rot_mult: float = 1.0,
+                   mix_src: Optional[torch.Tensor] = None, mix_col: int = 0,
+                   mix_lam: Optional[torch.Tensor] = None):
     """Take columns [col, col + n_heads*head_dim) of src [T, L]; RMS-norm
-    the first ``norm_cols`` of them together (weight ``norm_w``, plain);
-    rotate dims [rot_off, rot_off + rot_dims) of every head by the token's
-    position (pairs (i, i + rot_dims/2), angle pos * freqs[i]); all in
-    fp32. Without ``pool`` returns the rows as fp32 [T, n_heads*head_dim];
-    with ``pool`` [pages, n_heads, PAGE, head_dim] scatters them to the
-    tokens' page rows in the pool's dtype and returns None."""
+    the first ``norm_cols`` of them together (weight ``norm_w``, plain) or,
+    with ``head_norm``, every head on its own with the one weight
+    [head_dim]; rotate dims [rot_off, rot_off + rot_dims) of every head by
+    the token's position (pairs (i, i + rot_dims/2), or (2i, 2i+1) with
+    ``interleaved``; angle pos * freqs[i]; cos and sin times ``rot_mult``);
+    with ``mix_src`` blend the result with the same token's columns
+    [mix_col, mix_col + N) of that tensor, (1 - lam) x + lam m with lam =
+    ``mix_lam`` (one fp32 element); all in fp32. Without ``pool`` returns
+    the rows as fp32 [T, n_heads*head_dim]; with ``pool``
+    [pages, n_heads, PAGE, head_dim] scatters them to the tokens' page rows
+    in the pool's dtype and returns None."""
     N = n_heads * head_dim
     T = src.shape[0]
     if src.is_cuda:
@@ -465,10 +505,15 @@ def norm_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
                               norm_w, int(norm_cols), float(eps),
                               int(rot_off), int(rot_dims), freqs,
                               meta.tok_seq, meta.tok_pos, meta.table, out,
-                              pool)
+                              pool, bool(head_norm), bool(interleaved),
+                              float(rot_mult), mix_src, int(mix_col),
+                              mix_lam)
         return out
     x = src[:, col:col + N].float()
-    if norm_w is not None:
+    if norm_w is not None and head_norm:
+        x = (_rms(x.reshape(T, n_heads, head_dim), eps)
+             * norm_w).reshape(T, N)
+    elif norm_w is not None:
         x = torch.cat([_rms(x[:, :norm_cols], eps) * norm_w,
                        x[:, norm_cols:]], 1)
     x = x.reshape(T, n_heads, head_dim).clone()
@@ -476,11 +521,21 @@ def norm_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
     if rot_dims:
         half = rot_dims // 2
         ang = pos.double().view(T, 1, 1) * freqs.double().view(1, 1, half)
-        c, s = torch.cos(ang).float(), torch.sin(ang).float()
-        u = x[:, :, rot_off:rot_off + half].clone()
-        v = x[:, :, rot_off + half:rot_off + rot_dims].clone()
-        x[:, :, rot_off:rot_off + half] = u * c - v * s
-        x[:, :, rot_off + half:rot_off + rot_dims] = v * c + u * s
+        c = (torch.cos(ang) * rot_mult).float()
+        s = (torch.sin(ang) * rot_mult).float()
+        if interleaved:
+            iu = slice(rot_off, rot_off + rot_dims, 2)
+            iv = slice(rot_off + 1, rot_off + rot_dims, 2)
+        else:
+            iu = slice(rot_off, rot_off + half)
+            iv = slice(rot_off + half, rot_off + rot_dims)
+        u, v = x[:, :, iu].clone(), x[:, :, iv].clone()
+        x[:, :, iu] = u * c - v * s
+        x[:, :, iv] = v * c + u * s
+    if mix_src is not None:
+        lam = mix_lam.float().reshape(())
+        x = (1.0 - lam) * x + lam * mix_src[
+            :, mix_col:mix_col + N].float().reshape(T, n_heads, head_dim)
     if pool is None:
         return x.reshape(T, N)
     page = meta.table.long()[meta.tok_seq.long(), pos // PAGE]
@@ -499,6 +554,10 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
                    talk: Optional[torch.Tensor] = None, v_cols: int = 0,
                    softcap: float = 0.0,
                    sink_logits: Optional[torch.Tensor] = None,
+                   chunk: int = 0, keep_first: int = 0,
+                   dist_bias: Optional[torch.Tensor] = None,
+                   gate: Optional[torch.Tensor] = None, gate_col: int = 0,
+                   gate_heads: bool = False,
                    out_dtype=torch.float32) -> torch.Tensor:
     """Causal attention of the step's tokens over their sequences' cached
     rows (the step's own rows already appended).
@@ -511,7 +570,14 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
     ``window`` > 0 keeps keys with 0 <= i - j < window; ``sink`` adds one
     to the softmax denominator, ``sink_logits`` [H] (fp32) adds
     exp(sink_logits[h]) instead (a keyless, valueless entry that is neither
-    scaled nor capped). Scores, weights and sums are fp32.
+    scaled nor capped). ``chunk`` > 0 (instead of a window) keeps the keys
+    of the query's own chunk, floor(j / chunk) = floor(i / chunk), chunks
+    counted from position 0; ``keep_first`` > 0 keeps keys j < keep_first
+    visible whatever the window or chunk says. ``dist_bias`` [H, n] (fp32)
+    adds dist_bias[h, min(i - j, n - 1)] to the scaled score. ``gate``
+    [T, L] multiplies the result by sigmoid of its columns from
+    ``gate_col``: one per output column, or one per head with
+    ``gate_heads``. Scores, weights and sums are fp32.
     Returns [T, H*V] in ``out_dtype``."""
     G, DK = kpool.shape[1], kpool.shape[3]
     V = vpool.shape[3] if vpool is not None else v_cols
@@ -530,11 +596,15 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
             return _ext().flex_attn_tiles(
                 q, kpool, vpool, meta.query_tiles(), meta.table, talk,
                 int(H), float(scale), int(window), bool(sink), int(V),
-                out_dtype == torch.float32, float(softcap), sink_logits)
+                out_dtype == torch.float32, float(softcap), sink_logits,
+                int(chunk), int(keep_first), dist_bias, gate, int(gate_col),
+                bool(gate_heads))
         # few rows over long key ranges (decoding): spread each row's
         # keys over several blocks so the chip is filled; a function of
         # the step's shape only
-        span = min(meta.max_kv, window) if window > 0 else meta.max_kv
+        span = meta.max_kv
+        if window > 0 or chunk > 0:
+            span = min(span, max(window, chunk) + keep_first)
         n_split = 1
         while (n_split < 16 and meta.T * H * n_split < 2048
                and span > 256 * n_split):
@@ -544,7 +614,9 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
                                      float(scale), int(window), bool(sink),
                                      int(V), out_dtype == torch.float32,
                                      n_split, 1 if meta.T * H <= 512 else 8,
-                                     float(softcap), sink_logits)
+                                     float(softcap), sink_logits, int(chunk),
+                                     int(keep_first), dist_bias, gate,
+                                     int(gate_col), bool(gate_heads))
     out = torch.empty(T, H, V)
     qf = q.view(T, H, DK)
     rep = H // G
@@ -566,9 +638,17 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
             sc = softcap * torch.tanh(sc / softcap)
         qpos = torch.arange(meta.pos0_h[b], L).view(-1, 1)
         kpos = torch.arange(L).view(1, -1)
-        hide = kpos > qpos
+        if dist_bias is not None:
+            d = (qpos - kpos).clamp(0, dist_bias.shape[1] - 1)
+            sc = sc + dist_bias[:, d]
+        hide = torch.zeros_like(kpos > qpos)
         if window > 0:
-            hide = hide | (qpos - kpos >= window)
+            hide = qpos - kpos >= window
+        elif chunk > 0:
+            hide = (kpos // chunk) != (qpos // chunk)
+        if keep_first > 0:
+            hide = hide & (kpos >= keep_first)
+        hide = hide | (kpos > qpos)
         sc = sc.masked_fill(hide, float("-inf"))
         m = sc.amax(-1, keepdim=True)
         if sink:
@@ -580,6 +660,10 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
         if sink:
             den = den + torch.exp(sl - m)
         out[t0:t1] = torch.einsum("htj,jhv->thv", e / den, vb)
+    if gate is not None:
+        n = H if gate_heads else H * V
+        g = torch.sigmoid(gate[:, gate_col:gate_col + n].float())
+        out = out * (g.view(T, H, 1) if gate_heads else g.view(T, H, V))
     return out.reshape(T, H * V).to(out_dtype)
 
 
@@ -799,6 +883,31 @@ def yarn_freqs(dims: int, base: float, scaling: Optional[dict], device):
     ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
     f = f / factor * ramp + f * (1.0 - ramp)
     return f.to(device), 0.1 * math.log(factor) + 1.0
+
+
+def log_distance_buckets(rows: int, far: float) -> List[int]:
+    """Bucket of every distance n = 0, 1, ... up to the first that falls
+    into the last bucket (all larger ones do too). With half = rows // 2:
+    n < half has its own bucket n; beyond, buckets grow geometrically,
+    half + floor(ln(n / half) / ln(far / half) * (rows - half)), capped at
+    rows - 1. Evaluated in float64 on the host."""
+    import math
+    half = rows // 2
+    if rows < 2 or far <= half:
+        raise ValueError("distance buckets need rows >= 2 and a far "
+                         "distance beyond rows // 2")
+    out = []
+    n = 0
+    while True:
+        if n < half:
+            b = n
+        else:
+            b = min(rows - 1, half + int(math.floor(
+                math.log(n / half) / math.log(far / half) * (rows - half))))
+        out.append(b)
+        if b == rows - 1:
+            return out
+        n += 1
 
 
 def ssd_scan(xbc: torch.Tensor, offs, dt_src: torch.Tensor, dt_col: int,
