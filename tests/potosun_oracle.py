@@ -76,16 +76,22 @@ def rotate_halves(x, pos, dims, base, scaling=None):
 
 
 # ----------------------------------------------------------------- masks
+# a layer without a mask (size None) sees every earlier position
 def sees_window_keep(i, j, size, keep):
-    return j <= i and (i - j < size or j < keep)
+    return j <= i and (size is None or i - j < size or j < keep)
 
 
 def sees_chunk(i, j, size):
-    return j <= i and i // size == j // size
+    return j <= i and (size is None or i // size == j // size)
 
 
 def sees_window(i, j, size):
-    return 0 <= i - j < size
+    return 0 <= i - j and (size is None or i - j < size)
+
+
+def mask_of(mc):
+    m = mc.get("mask") or {}
+    return m.get("size"), m.get("keep_first", 0)
 
 
 def distance_bucket(n, rows, far):
@@ -115,7 +121,7 @@ def mix_values(v, mc, P, vmix):
         vmix["first"] = v
         return v
     lam = float(P["vmix"])
-    return (1.0 - lam) * v + lam * vmix["first"]
+    return (1.0 - lam) * v + lam * vmix["first"].reshape(v.shape)
 
 
 # ---------------------------------------------------------------- mixers
@@ -128,8 +134,7 @@ def biased_attention(h, P, mc, eps, vmix):
     k = rms((h @ P["k"].T).reshape(T, G, D), eps) * P["k.norm"]
     v = mix_values((h @ P["v"].T).reshape(T, G, V), mc, P, vmix)
     rel = P["rel"]
-    size = mc["mask"]["size"]
-    keep = mc["mask"].get("keep_first", 0)
+    size, keep = mask_of(mc)
     o = np.zeros((T, H, V))
     for i in range(T):
         js = [j for j in range(i + 1) if sees_window_keep(i, j, size, keep)]
@@ -157,7 +162,7 @@ def chunked_attention(h, P, mc, eps, vmix):
     k = np.stack([rotate_interleaved(k[t], t, rot["dims"], rot["base"])
                   for t in range(T)])
     v = mix_values((h @ P["v"].T).reshape(T, G, V), mc, P, vmix)
-    size = mc["mask"]["size"]
+    size, _ = mask_of(mc)
     o = np.zeros((T, H, V))
     for i in range(T):
         js = [j for j in range(i + 1) if sees_chunk(i, j, size)]
@@ -188,7 +193,7 @@ def latent_attention(h, P, mc, eps):
     ku = (c @ P["uk"].T).reshape(T, H, D)
     vv = (c @ P["uv"].T).reshape(T, H, V)
     gate = sigmoid(h @ P["g"].T)                       # [T, H]
-    size = mc["mask"]["size"]
+    size, _ = mask_of(mc)
     o = np.zeros((T, H, V))
     for i in range(T):
         js = [j for j in range(i + 1) if sees_window(i, j, size)]
@@ -210,7 +215,7 @@ def forward(cfg, W, tokens, layer_out=None):
     W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
     eps = cfg["norm"]["eps"]
     tokens = np.asarray(tokens, dtype=np.int64)
-    x = W["embed"][tokens] * cfg["embedding"]["scale"]
+    x = W["embed"][tokens] * (cfg.get("embedding") or {}).get("scale", 1.0)
     vmix = {}
     for i, lc in enumerate(cfg["layers"]):
         mc = lc["mixer"]
