@@ -49,11 +49,13 @@ def parse_args():
                         "beside an equal-size Qwen3-MoE-shaped model")
     p.add_argument("--sizes", default="w1024,w2048",
                    help="layered mode: comma list of size presets")
-    p.add_argument("--family", choices=["kepusun", "senulix", "dizepel"],
+    p.add_argument("--family",
+                   choices=["kepusun", "senulix", "dizepel", "potosun"],
                    default="kepusun",
                    help="layered mode: which layered family to time "
                         "(senulix, dizepel: beside an equal-size dense GQA "
-                        "decoder)")
+                        "decoder; potosun: beside an equal-size Senulix "
+                        "model)")
     p.add_argument("--dp", type=int, default=1,
                    help="data-parallel replicas (train mode; world=dp*pp)")
     return p.parse_args()
@@ -254,6 +256,57 @@ def dizepel_configs(z):
     return diz, ref
 
 
+POTOSUN_SIZES = {
+    # layers: latent, biased window, biased window, chunked, latent, biased
+    "w1024": dict(width=1024, heads=8, kv=2, dim=128, rot=64, rank=192,
+                  window=1024, keep=64, chunk=1024, rows=32, far=4096,
+                  ff=4096, side=32, vocab=32000, batch=8, prompt=2048),
+    "w2048": dict(width=2048, heads=16, kv=4, dim=128, rot=64, rank=192,
+                  window=1024, keep=64, chunk=1024, rows=32, far=4096,
+                  ff=8192, side=64, vocab=32000, batch=8, prompt=2048),
+    "tiny": dict(width=128, heads=2, kv=1, dim=32, rot=16, rank=48,
+                 window=64, keep=4, chunk=48, rows=8, far=100, ff=256,
+                 side=8, vocab=512, batch=2, prompt=96),
+}
+
+
+def potosun_configs(z):
+    """(Potosun config, Senulix config) of a preset: same width, depth,
+    vocabulary, head count, head sizes, latent rank and window; Potosun's
+    gated three-matrix feed-forward gets 2/3 of the width of Senulix's
+    two-matrix one, which equalises their parameters."""
+    from tensorlink_amd.models.potosun import PotosunConfig
+    H, D = z["heads"], z["dim"]
+    ff = (2 * z["ff"] // 3 + 63) // 64 * 64
+    mlp = {"kind": "dense", "ff": ff}
+    la = {"heads": H, "dim": D, "rot_dim": z["rot"], "vdim": D,
+          "kv_rank": z["rank"], "scale": (D + z["rot"]) ** -0.5,
+          "rot": {"dims": z["rot"], "base": 10000.0,
+                  "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0,
+                              "slow": 2.0}},
+          "mask": {"size": z["window"]}}
+    ba = {"heads": H, "kv_heads": z["kv"], "dim": D, "vdim": D,
+          "scale": D ** -0.5, "bias_max": z["far"], "bias_rows": z["rows"],
+          "mask": {"size": z["window"], "keep_first": z["keep"]},
+          "v_mix": True}
+    ca = {"heads": H, "kv_heads": z["kv"], "dim": D, "vdim": D,
+          "scale": D ** -0.5, "rot": {"dims": D, "base": 1000000.0},
+          "mask": {"size": z["chunk"]}, "v_mix": True}
+    layers = [{"type": "latent_attention", "mixer": la, "mlp": mlp},
+              {"type": "attention", "mixer": ba, "mlp": mlp},
+              {"type": "attention", "mixer": ba, "mlp": mlp},
+              {"type": "attention_2", "mixer": ca, "mlp": mlp},
+              {"type": "latent_attention", "mixer": la, "mlp": mlp},
+              {"type": "attention", "mixer": ba, "mlp": mlp}]
+    pot = PotosunConfig.from_dict({
+        "architecture": "Potosun", "vocab": z["vocab"], "width": z["width"],
+        "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+        "logit_softcap": 30.0, "layers": layers},
+        name="potosun-" + str(z["width"]))
+    sen, _ = senulix_configs(z)
+    return pot, sen
+
+
 @torch.no_grad()
 def run_layered(args, device, use_gpu):
     """Prefill and decode tokens/s of the Kepusun family beside the
@@ -303,7 +356,17 @@ def run_layered(args, device, use_gpu):
         return out
 
     for name in args.sizes.split(","):
-        if args.family == "dizepel":
+        if args.family == "potosun":
+            z = POTOSUN_SIZES[name]
+            pot, sen = potosun_configs(z)
+            B, S = z["batch"], z["prompt"]
+            only = os.environ.get("TL_BENCH_ONLY")     # profile one model
+            res = {}
+            if only in (None, "potosun"):
+                res["potosun"] = measure(pot, B, S)
+            if only in (None, "senulix"):
+                res["senulix"] = measure(sen, B, S)
+        elif args.family == "dizepel":
             z = DIZEPEL_SIZES[name]
             diz, ref = dizepel_configs(z)
             B, S = z["batch"], z["prompt"]

@@ -247,11 +247,9 @@ class PotosunStageModel(LayeredStage):
             if layer.mlp is not None:
                 h = mx.add_rms(X, y, layer.norm2.w32(), eps, dtype)
                 y = layer.mlp(h)
-        if scale != 1.0:
-            X *= scale
-        if y is not None:
-            X += y
-            if self.layer_sums is not None:
+        if y is not None or scale != 1.0:
+            mx.add_rms(X, y, None, eps, dtype, x_scale=scale)
+            if self.layer_sums is not None and y is not None:
                 self.layer_sums.append(X.clone())
         if kv_cache is not None:
             kv_cache.advance(S)

@@ -140,24 +140,30 @@ Tensor rms_scale(Tensor x, Tensor w, double eps, bool one_plus,
   return out;
 }
 
-// X (*= x_scale) += y; returns rms(X) * w in the serving dtype
-Tensor add_rms(Tensor X, c10::optional<Tensor> y, Tensor w, double eps,
-               double x_scale, bool out_f32) {
+// X (*= x_scale) += y; returns rms(X) * w in the serving dtype, or,
+// without a weight, X itself after the add
+Tensor add_rms(Tensor X, c10::optional<Tensor> y, c10::optional<Tensor> w,
+               double eps, double x_scale, bool out_f32) {
   SEQ_F32(X);
-  SEQ_F32(w);
-  TORCH_CHECK(X.dim() == 2 && w.numel() == X.size(1),
-              "X must be [T, W], the norm weight [W]");
+  TORCH_CHECK(X.dim() == 2, "X must be [T, W]");
+  if (w.has_value()) {
+    SEQ_F32(w.value());
+    TORCH_CHECK(w->numel() == X.size(1), "the norm weight must be [W]");
+  }
   if (y.has_value()) {
     SEQ_IN(y.value());
     TORCH_CHECK(y->sizes() == X.sizes(), "y must be [T, W]");
     TORCH_CHECK(act_is_f32(y.value()) == (out_f32 ? 1 : 0),
                 "y / output dtype mismatch");
   }
-  auto h = torch::empty(
-      X.sizes(), X.options().dtype(out_f32 ? torch::kFloat : torch::kBFloat16));
+  Tensor h = X;
+  if (w.has_value())
+    h = torch::empty(X.sizes(), X.options().dtype(out_f32 ? torch::kFloat
+                                                          : torch::kBFloat16));
   tl_add_rms(X.data_ptr(), y.has_value() ? y->data_ptr() : nullptr,
-             w.data_ptr(), h.data_ptr(), X.size(0), (int)X.size(1), (float)eps,
-             (float)x_scale, out_f32 ? 1 : 0, seq_stream());
+             w.has_value() ? w->data_ptr() : nullptr,
+             w.has_value() ? h.data_ptr() : nullptr, X.size(0), (int)X.size(1),
+             (float)eps, (float)x_scale, out_f32 ? 1 : 0, seq_stream());
   return h;
 }
 

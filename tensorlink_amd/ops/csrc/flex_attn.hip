@@ -133,6 +133,14 @@ __global__ __launch_bounds__(BLOCK) void norm_rope_rows_kernel(
 }
 
 // -------------------------------------------------------------- attention
+// lanes that cover one value row of V columns with 16-byte loads: the
+// power of two at or above V / 8
+__host__ __device__ inline int vec_lanes(int V) {
+  int n = 1;
+  while (n * 8 < V) n <<= 1;
+  return n;
+}
+
 // sigmoid of the output gate of column c of head h of token t; 1 without
 DEVINLINE float out_gate(const TlFlexExtra& ex, int64_t t, int h, int V,
                          int c) {
@@ -186,9 +194,10 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
   __syncthreads();
 
   // VR == 0: value rows are fetched with 16-byte loads (bf16 pools, value
-  // size 8 * 2^k): CPR lanes cover one row, so one load instruction brings
-  // 64 / CPR rows; a lane accumulates 8 columns for the keys of its row
-  // group and the row groups meet through shuffles at the end
+  // size a multiple of 8): CPR lanes (the power of two at or above V / 8;
+  // those beyond the row stay idle) cover one row, so one load instruction
+  // brings 64 / CPR rows; a lane accumulates 8 columns for the keys of its
+  // row group and the row groups meet through shuffles at the end
   constexpr int AC = VR == 0 ? 8 : VR;
   float m[HB], l[HB], a[HB][AC];
 #pragma unroll
@@ -263,21 +272,22 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
     const int jb = max(0, rlo - j0), je = min(WAVE_SIZE, rhi + 1 - j0);
     const TK* vtile = vpool + (page_row + (int64_t)g0 * PAGE) * vld;
     if constexpr (VR == 0) {
-      const int CPR = V >> 3, KGR = WAVE_SIZE / CPR;
+      const int CPR = vec_lanes(V), KGR = WAVE_SIZE / CPR;
       const int cc = lane & (CPR - 1), kg = lane / CPR;
+      const bool col_on = cc * 8 < V;
       for (int jj0 = jb; jj0 < je; jj0 += 4 * KGR) {
         bf16x8 vv[4];
         int jk[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           jk[u] = jj0 + u * KGR + kg;
-          if (jk[u] < je)
+          if (jk[u] < je && col_on)
             vv[u] = *reinterpret_cast<const bf16x8*>(
                 vtile + (int64_t)jk[u] * vld + cc * 8);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const bool on = jk[u] < je;
+          const bool on = jk[u] < je && col_on;
           const int src = min(jk[u], WAVE_SIZE - 1);
 #pragma unroll
           for (int b = 0; b < HB; ++b) {
@@ -325,13 +335,14 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
       stat[(wave * HB + b) * 2 + 1] = l[b];
     }
     if constexpr (VR == 0) {
-      const int CPR = V >> 3;
+      const int CPR = vec_lanes(V);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         float s = a[b][e];
         for (int off = CPR; off < WAVE_SIZE; off <<= 1)
           s += __shfl_xor(s, off, WAVE_SIZE);
-        if (lane < CPR) accs[(wave * HB + b) * V + lane * 8 + e] = s;
+        if (lane < CPR && lane * 8 < V)
+          accs[(wave * HB + b) * V + lane * 8 + e] = s;
       }
     } else {
 #pragma unroll
@@ -530,10 +541,10 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
   else if (hb == 4) { TL_FA_V(TT, 4) } \
   else if (hb == 2) { TL_FA_V(TT, 2) } \
   else { TL_FA_V(TT, 1) }
-  // 16-byte value loads: bf16 rows of 8 * 2^k columns, 16-byte aligned
-  const int cpr = V / 8;
-  const bool vec = !pool_f32 && V % 8 == 0 && cpr >= 1 && cpr <= WAVE_SIZE &&
-                   (cpr & (cpr - 1)) == 0 && vld % 8 == 0 && !no_vec;
+  // 16-byte value loads: bf16 rows of a multiple of 8 columns, 16-byte
+  // aligned
+  const bool vec = !pool_f32 && V % 8 == 0 && V >= 8 &&
+                   vec_lanes(V) <= WAVE_SIZE && vld % 8 == 0 && !no_vec;
   if (pool_f32) {
     TL_FA_H(float)
   } else if (vec) {

@@ -62,7 +62,7 @@ __global__ __launch_bounds__(BLOCK) void postnorm_add_kernel(
   }
 }
 
-// X += y (if given); h = X / rms(X) * w in the serving dtype
+// X += y (if given); h = X / rms(X) * w in the serving dtype (no w: no h)
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void add_rms_kernel(
     float* __restrict__ X, const T* __restrict__ y,
@@ -78,6 +78,7 @@ __global__ __launch_bounds__(BLOCK) void add_rms_kernel(
     if (y || x_scale != 1.f) xr[c] = v;
     ss += v * v;
   }
+  if (!w) return;                 // the residual add alone
   const float tot = block_reduce_sum<NW>(ss, red);
   const float rn = 1.0f / sqrtf(tot / (float)W + eps);
   // a thread reads back only what it wrote itself

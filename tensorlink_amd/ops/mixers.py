@@ -432,23 +432,25 @@ def soft_cap_(z: torch.Tensor, cap: float) -> torch.Tensor:
     return z.copy_(cap * torch.tanh(z / cap))
 
 
-def add_rms(X: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor,
-            eps: float, out_dtype=torch.float32,
+def add_rms(X: torch.Tensor, y: Optional[torch.Tensor],
+            w: Optional[torch.Tensor], eps: float, out_dtype=torch.float32,
             x_scale: float = 1.0) -> torch.Tensor:
     """Pre-norm residual step, in place on the fp32 residual X [T, W]:
     X <- X * x_scale + y (``y`` = the previous sublayer's output, or None),
-    then returns the next sublayer's input X / rms(X) * w in ``out_dtype``.
-    Sum, statistic and scaling are fp32."""
-    assert X.dtype == torch.float32 and w.dtype == torch.float32
+    then returns the next sublayer's input X / rms(X) * w in ``out_dtype``;
+    without ``w`` (after the last sublayer) only the add is done and X is
+    returned. Sum, statistic and scaling are fp32."""
+    assert X.dtype == torch.float32
+    assert w is None or w.dtype == torch.float32
     if X.is_cuda:
-        return _ext().add_rms(X, None if y is None else y.contiguous(), w,
-                              float(eps), float(x_scale),
-                              out_dtype == torch.float32)
+        return _ext().add_rms(
+            X, None if y is None else y.contiguous(), w, float(eps),
+            float(x_scale), out_dtype == torch.float32)
     if x_scale != 1.0:
         X *= x_scale
     if y is not None:
         X += y.float()
-    return (_rms(X, eps) * w).to(out_dtype)
+    return X if w is None else (_rms(X, eps) * w).to(out_dtype)
 
 
 def gelu_gate(p: torch.Tensor, tanh_form: bool = True) -> torch.Tensor:
