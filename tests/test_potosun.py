@@ -153,6 +153,24 @@ def cfg_tiles():
                  "mlp": FF}]}
 
 
+def cfg_odd():
+    """Sizes that are multiples of 2 at most: width, feed-forward, vocabulary,
+    head sizes, latent rank, table rows; three query heads per key head."""
+    return {"architecture": "Potosun", "vocab": 37, "width": 36,
+            "norm": {"eps": 1e-5}, "embedding": {"scale": 2.5},
+            "logit_softcap": 9.0, "layers": [
+                {"type": "attention",
+                 "mixer": att(3, 1, 10, 6, 21, keep=2, rows=5, far=17,
+                              v_mix=True),
+                 "mlp": {"kind": "dense", "ff": 50}},
+                {"type": "latent_attention",
+                 "mixer": lat(3, 10, 6, 14, 12, window=19, scaling=YARN),
+                 "mlp": {"kind": "dense", "ff": 50}},
+                {"type": "attention_2",
+                 "mixer": att2(6, 1, 6, 6, 27, 2, v_mix=True),
+                 "mlp": None}]}
+
+
 def mixer_weights(lc, w, rnd):
     """Checkpoint tensors of one mixer (names without the layer prefix)."""
     mc, P = lc["mixer"], {}
@@ -849,7 +867,7 @@ def test_tile_kernel_against_row_kernel_and_plain():
 
 
 # ---------------------------------------------------------- whole model
-CFGS = [cfg_mixed, cfg_ones, cfg_wide, cfg_tiles]
+CFGS = [cfg_mixed, cfg_ones, cfg_wide, cfg_tiles, cfg_odd]
 
 
 @pytest.mark.parametrize("cfg_fn", CFGS, ids=lambda f: f.__name__)
