@@ -982,6 +982,58 @@ def test_greedy_generation(tmp_path_factory, device, dtype):
     assert out[0].tolist()[:keep] == want[0][:keep]
 
 
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_trace_runner(tmp_path_factory, tmp_path, device, dtype):
+    """bin/trace_run as a user starts it: steps on standard input, three
+    requests through a pool of three pages (the first ends before the
+    third starts), portions beside single tokens, logits files for the
+    wanted places only, a line per step."""
+    import subprocess
+    import sys
+    _, P, cfg = model(tmp_path_factory, cfg_mixed, "cpu", torch.float32)
+    d = _CACHE[("cfg_mixed", 0)][0]
+    reqs = {"a": tokens(cfg, 100, 11), "b": tokens(cfg, 130, 12),
+            "c": tokens(cfg, 90, 13)}
+    want = {k: oracle(cfg, P, v) for k, v in reqs.items()}
+    plan = [[("a", 60, [0, 59])], [("a", 39, [38]), ("b", 2, [])],
+            [("a", 1, [0]), ("b", 127, [5, 126])], [("b", 1, [0]),
+                                                    ("c", 88, [87])],
+            [("c", 1, [])], [("c", 1, [0])]]
+    at = {k: 0 for k in reqs}
+    lines, rows = [], []
+    for n, step in enumerate(plan):
+        entries, end, asked = [], [], []
+        for rid, cnt, wanted in step:
+            entries.append({"id": rid, "want": wanted,
+                            "tokens": reqs[rid][at[rid]:at[rid] + cnt]})
+            asked += [(rid, at[rid] + k) for k in wanted]
+            at[rid] += cnt
+            if at[rid] == len(reqs[rid]):
+                end.append(rid)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+        rows.append(asked)
+    exe = os.path.join(os.path.dirname(os.path.dirname(
+        os.path.abspath(__file__))), "bin", "trace_run")
+    out = str(tmp_path / "out")
+    r = subprocess.run(
+        [sys.executable, exe, "--model", d, "--out", out, "--device", device,
+         "--dtype", "float32" if dtype == torch.float32 else "bfloat16",
+         "--max-tokens", "320"], input="\n".join(lines) + "\n",
+        capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    done = [ln for ln in r.stdout.splitlines() if ln.startswith("done ")]
+    assert done == ["done %d" % n for n in range(len(plan))]
+    for n, asked in enumerate(rows):
+        f = os.path.join(out, "%d.f32" % n)
+        if not asked:
+            assert not os.path.exists(f)
+            continue
+        got = torch.from_numpy(np.fromfile(f, dtype="<f4").reshape(
+            len(asked), cfg["vocab"]).copy())
+        ref = torch.stack([want[rid][p] for rid, p in asked])
+        assert close(got, ref, dtype), n
+
+
 def random_cfg(rng):
     """A random model of the design: 2-5 layers in any order, 1-9 heads,
     head sizes from 8 to 136 (below, at and above a wave's 64 columns, not
