@@ -585,10 +585,12 @@ void register_seq_ops(pybind11::module& mod) {
           "GELU (erf or tanh form) times an optional gathered table slice");
   mod.def("soft_cap_", &soft_cap_, "cap * tanh(z / cap) in place");
   mod.def("norm_rope_rows", &norm_rope_rows,
-          "RMS norm + rotate-half positions on projection rows, dense or "
+          "RMS norm (whole range or per head) + rotary positions (halves or "
+          "interleaved) + optional blend on projection rows, dense or "
           "scattered into a page pool");
   mod.def("flex_attn_rows", &flex_attn_rows,
-          "paged softmax attention: window, sink, score mixing, latent rows");
+          "paged softmax attention: window / chunk / kept prefix, sink, "
+          "distance bias, score mixing, latent rows, output gate");
   mod.def("flex_attn_tiles_ok", &flex_attn_tiles_ok,
           "whether the MFMA tile kernel serves a shape");
   mod.def("flex_attn_tiles", &flex_attn_tiles,

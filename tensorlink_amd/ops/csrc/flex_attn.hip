@@ -9,6 +9,11 @@
 // the latent part of a latent row), rotate-half positions on a sub-range of
 // every head, then either a dense fp32 copy (queries) or a scatter into the
 // tokens' page rows (keys, values, latents). Angles are pos * f_i in double.
+// Options: the norm per head over the head's columns with one shared weight,
+// rotation pairs (2i, 2i+1) instead of halves, a multiplier on cos and sin
+// (scaled rotations), and a blend (1 - lam) x + lam m with the same token's
+// columns of another projection (value mixing across layers) before the
+// row is written.
 //
 // tl_flex_attn_rows serves one query token and HB query heads of one key
 // group per block. Each of the four waves strides over 64-key tiles of the
